@@ -129,7 +129,7 @@ __global__ __launch_bounds__(NWV * 64, (NWV == 4 && (MT > 4 || TS == 2 || MODE =
     }
 // SiLU-gate form up to 192 tokens (BQ = 2): the B fragments of k-step kk+1 are requested BEFORE the MFMAs of k-step kk (two
 // register sets, pinned by scheduling barriers). Left to itself the compiler issues each pair of ds_reads right in front of
-// the two MFMAs that consume them (`dd w M w M` in tools/isa_mix.py --seq). Measured (profiles/r06d_gemm_wide_pipe_ab.jsonl):
+// the two MFMAs that consume them. Measured (profiles/r06d_gemm_wide_pipe_ab.jsonl):
 // up/gate + SiLU 51.5 vs 55.2 us at 96 tokens, 54.1 vs 55.9 at 128, 71.0 vs 76.5 at 192; the partial-slab kernels (qkv, o,
 // down) are 1-4 us SLOWER with it at 256 tokens and level below, and keep one set.
 #define SWL_W_PROCESS(slot, buf)                                                                      \
