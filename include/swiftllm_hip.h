@@ -35,6 +35,7 @@ extern "C" {
 
 #define SWL_F16 0
 #define SWL_BF16 1
+#define SWL_F32 2 /* only the operators that say so accept it */
 
 #define SWL_OK 0
 #define SWL_ERR_BAD_ARG (-1)     /* null pointer, negative size, misaligned pointer/stride          */
@@ -488,6 +489,59 @@ int swl_decode_engine_step(void *resid_out, const void *w_stream, const void *no
                            int32_t hidden, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                            int32_t ffn_inter_dim, int32_t max_blocks_per_seq, float eps, float softmax_scale,
                            int32_t flags, int32_t dtype, swl_stream_t stream);
+
+/* ---- fp32 residual stream: embedding with learned positions, LayerNorm, fused sandwich-norm step ------------------
+ * (no counterpart in the reference, which serves LLaMA only; used by the Kekapel model.) dtype may be SWL_F32.
+ * swl_embed_pos:     x[t] = embed[tokens[t]] * scale + pos[positions[t]] in fp32; x0 (may be NULL) gets a copy.
+ * swl_layernorm:     out[r] = (x[i] - mean) / sqrt(var + eps) * w + b of row i = row_idx ? row_idx[r] : r (fp32 stats,
+ *                    var = mean of squared deviations); out in dtype, x / w / b fp32.
+ * swl_add_layernorm: x += mult * LN(y; w1, b1) (if y) + x0 (if x0) + step (if step, a [width] vector);
+ *                    out = LN(x; w2, b2) (if out). y / out in dtype. */
+int swl_embed_pos(float *x, float *x0, const void *embed, const void *pos, const int32_t *tokens,
+                  const int32_t *positions, float scale, int64_t num_tokens, int32_t width, int32_t dtype,
+                  swl_stream_t stream);
+int swl_layernorm(void *out, const float *x, const int32_t *row_idx, const float *w, const float *b, float eps,
+                  int64_t num_rows, int32_t width, int32_t dtype, swl_stream_t stream);
+int swl_add_layernorm(float *x, const void *y, float mult, const float *w1, const float *b1, const float *x0,
+                      const float *step, void *out, const float *w2, const float *b2, float eps, int64_t num_tokens,
+                      int32_t width, int32_t dtype, swl_stream_t stream);
+
+/* ---- per-head q/k RMS norm + paged KV store ---------------------------------------------------------------------------
+ * qkv[T, tok_stride] = [q heads | k heads | v heads] of one fused projection. q heads are normalised in place (weight q_w
+ * [dim], shared by the heads); k heads are normalised (k_w) into the K pool (block b = [kv_heads, 16, dim] at k_cache + b * block_stride
+ * elements); v heads are copied into the V pool (block b = [kv_heads, 16, vdim] at v_cache + b * block_stride), block
+ * block_table[tok_seq[t]][tok_pos[t] / 16], slot tok_pos[t] % 16.
+ * k_cache == NULL: only the query norm (memory-profiling runs). dtype may be SWL_F32. */
+int swl_qknorm_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_cache, void *v_cache,
+                        const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos, int64_t num_tokens,
+                        int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t tok_stride,
+                        int32_t max_blocks_per_seq, int64_t block_stride, float eps, int32_t dtype, swl_stream_t stream);
+
+/* ---- sliding-window attention with soft-capping and pre-softmax head mixing over the paged pool -----------------------
+ * out[T, H * vdim]; token t attends keys [max(0, p - window + 1), p] of its sequence (window 0: all), p = tok_pos[t];
+ * score = softcap * tanh(q.k * scale / softcap) (softcap 0: none), mixed over heads by talk[H, H] (fp32), softmax, values.
+ * H <= 32, H * vdim <= 8192. dtype may be SWL_F32. */
+int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
+                    const int32_t *tok_seq, const int32_t *tok_pos, const float *talk, int64_t num_tokens,
+                    int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride,
+                    int32_t window, float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride,
+                    int32_t dtype, swl_stream_t stream);
+
+/* ---- PolyNorm activation: out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row ---------- */
+int swl_polynorm(void *out, const void *z, float a, float b, float c, float e, float eps, int64_t num_rows, int32_t ff,
+                 int32_t dtype, swl_stream_t stream);
+
+/* ---- mixture of experts ---------------------------------------------------------------------------------------------------
+ * swl_moe_route: idx_out[T, top] / w_out[T, top] = the top experts of fp32 logits router[experts, width] h + bias and the
+ * softmax over the chosen logits. swl_moe_gate_up: y[T * top, ff] = clamped gated unit of expert idx[a] on token a / top;
+ * gate_up [experts, 2 ff, width] = gate rows then up rows. swl_moe_down_combine: out[T, width] = sum_j w[t][j] down[e_j] y.
+ * dtype may be SWL_F32. */
+int swl_moe_route(int32_t *idx_out, float *w_out, const void *h, const float *router, const float *bias,
+                  int64_t num_tokens, int32_t width, int32_t experts, int32_t top, int32_t dtype, swl_stream_t stream);
+int swl_moe_gate_up(void *y, const void *h, const void *gate_up, const int32_t *expert_idx, int64_t num_tokens,
+                    int32_t width, int32_t ff, int32_t top, float limit, int32_t dtype, swl_stream_t stream);
+int swl_moe_down_combine(void *out, const void *y, const void *down, const int32_t *expert_idx, const float *expert_w,
+                         int64_t num_tokens, int32_t width, int32_t ff, int32_t top, int32_t dtype, swl_stream_t stream);
 
 #ifdef __cplusplus
 }

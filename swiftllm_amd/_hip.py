@@ -20,6 +20,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", _LI
 
 SWL_F16 = 0
 SWL_BF16 = 1
+SWL_F32 = 2     # only the operators that say so accept it
 ABI_VERSION = 1
 
 _P = ctypes.c_void_p
@@ -92,6 +93,17 @@ SIGNATURES = {
     "swl_decode_engine_reset": [_P, ctypes.c_size_t, _P],
     "swl_decode_engine_step": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, _P, _P, _I32, _I32,
                                _I32, _I32, _I32, _I32, _I32, _F32, _F32, _I32, _I32, _P],
+    "swl_embed_pos": [_P, _P, _P, _P, _P, _P, _F32, _I64, _I32, _I32, _P],
+    "swl_layernorm": [_P, _P, _P, _P, _P, _F32, _I64, _I32, _I32, _P],
+    "swl_add_layernorm": [_P, _P, _F32, _P, _P, _P, _P, _P, _P, _P, _F32, _I64, _I32, _I32, _P],
+    "swl_qknorm_store_kv": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _I64, _F32, _I32,
+                            _P],
+    "swl_window_attn": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32, _I32,
+                        _I64, _I32, _P],
+    "swl_polynorm": [_P, _P, _F32, _F32, _F32, _F32, _F32, _I64, _I32, _I32, _P],
+    "swl_moe_route": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
+    "swl_moe_gate_up": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _P],
+    "swl_moe_down_combine": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
 }
 # Entry points that do not follow the "int rc = f(...)" convention.
 _SPECIAL = {
@@ -141,14 +153,18 @@ def load():
             lib = ctypes.CDLL(path)
         except OSError as e:
             raise HipLibraryError(f"cannot load {path}: {e}") from e
+        # A library built for one model family (csrc/build.py: `only`) lacks the other families' entry points: those stay
+        # unbound and `call` says how to get them.
         for name, argtypes in SIGNATURES.items():
-            fn = getattr(lib, name)
-            fn.argtypes = argtypes
-            fn.restype = _I32
+            fn = getattr(lib, name, None)
+            if fn is not None:
+                fn.argtypes = argtypes
+                fn.restype = _I32
         for name, (argtypes, restype) in _SPECIAL.items():
-            fn = getattr(lib, name)
-            fn.argtypes = argtypes
-            fn.restype = restype
+            fn = getattr(lib, name, None)
+            if fn is not None:
+                fn.argtypes = argtypes
+                fn.restype = restype
         got = lib.swl_abi_version()
         if got != ABI_VERSION:
             raise HipLibraryError(f"{path} has ABI version {got}, this package needs {ABI_VERSION}; rebuild")
@@ -163,7 +179,10 @@ def is_available() -> bool:
 
 def call(name: str, *args) -> None:
     """Invoke `name`; map a non-zero return code to HipLibraryError (a RuntimeError)."""
-    rc = getattr(load(), name)(*args)
+    fn = getattr(load(), name, None)
+    if fn is None:
+        raise HipLibraryError(f"{library_path()} was built without {name}: run `python -m swiftllm_amd.csrc.build`")
+    rc = fn(*args)
     if rc != 0:
         msg = load().swl_strerror(rc).decode()
         raise HipLibraryError(f"{name} failed with code {rc}: {msg}")
@@ -180,6 +199,11 @@ def dtype_code(dtype: torch.dtype) -> int:
     if dtype == torch.bfloat16:
         return SWL_BF16
     raise TypeError(f"libswiftllm_hip supports float16 and bfloat16, got {dtype}")
+
+
+def dtype_code3(dtype: torch.dtype) -> int:
+    """Code for the operators that also run in true fp32."""
+    return SWL_F32 if dtype == torch.float32 else dtype_code(dtype)
 
 
 def ptr(t) -> int:

@@ -29,14 +29,29 @@ SOURCES = [
     "gemm_rows.hip",
     "argmax.hip",
     "decode_engine.hip",
+    "layernorm.hip",
+    "qknorm_kv.hip",
+    "window_attn.hip",
+    "polynorm.hip",
+    "moe.hip",
 ]
+# What a model family's worker calls (the shared pieces included): `build(only=MODEL_SOURCES[...])` compiles just these, so
+# that the first use from a fresh checkout does not pay for kernels the model never launches. A later full build compiles
+# the rest and links everything.
+_SHARED = ["swap_blocks.hip", "block_table.hip", "argmax.hip", "gemm_skinny.hip", "gemm_wide.hip"]
+MODEL_SOURCES = {
+    "llama": list(SOURCES[:14]),
+    "Kekapel": _SHARED + ["layernorm.hip", "qknorm_kv.hip", "window_attn.hip", "polynorm.hip", "moe.hip"],
+}
 HEADERS = ["swl_common.h", "attend_block.h", os.path.join(ROOT, "include", "swiftllm_hip.h")]
 LIB = os.path.join(HERE, "libswiftllm_hip.so")
 OBJ_DIR = os.path.join(HERE, "build")
 ARCH = "gfx950"
 # -ffp-contract=off: the reference's rounding points (fp16 mul, then fp16 add) must not be fused.
 CXXFLAGS = [f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wall",
-            "-Wno-unused-function"]
+            "-Wno-unused-function",
+            # the compiler may not form packed-fp32 VALU ops from scalar float code
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def _hipcc() -> str:
@@ -53,17 +68,18 @@ def _newer(target: str, deps) -> bool:
     return all(os.path.getmtime(d) <= t for d in deps)
 
 
-def build(force: bool = False, jobs: int = 0, verbose: bool = True, tag: str = "", defines=(), swap=None) -> str:
+def build(force: bool = False, jobs: int = 0, verbose: bool = True, tag: str = "", defines=(), swap=None,
+          only=None) -> str:
     """Build the library. `tag` + `defines` (-D macros) / `swap` build an EXPERIMENT variant next to it
     (libswiftllm_hip_<tag>.so; its objects go to the system temp directory, not into the tree that ships to the GPU
     box): tools/ select one with SWIFTLLM_HIP_LIB to A/B a kernel on the GPU box without touching the product library."""
     hipcc = _hipcc()
     obj_dir = os.path.join(tempfile.gettempdir(), "swiftllm_hip_variants", tag) if tag else OBJ_DIR
     lib = os.path.join(HERE, f"libswiftllm_hip_{tag}.so") if tag else LIB
-    return _build(hipcc, obj_dir, lib, [f"-D{d}" for d in defines], force, jobs, verbose, swap or {})
+    return _build(hipcc, obj_dir, lib, [f"-D{d}" for d in defines], force, jobs, verbose, swap or {}, only)
 
 
-def _build(hipcc, OBJ_DIR, LIB, extra, force, jobs, verbose, swap) -> str:
+def _build(hipcc, OBJ_DIR, LIB, extra, force, jobs, verbose, swap, only=None) -> str:
     """`swap`: {source name: replacement path} — an experiment variant may compile another file in a source's place
     (e.g. an older revision of one kernel for an A/B run)."""
     os.makedirs(OBJ_DIR, exist_ok=True)
@@ -73,8 +89,13 @@ def _build(hipcc, OBJ_DIR, LIB, extra, force, jobs, verbose, swap) -> str:
     for src in SOURCES:
         src_path = swap.get(src, os.path.join(HERE, src))
         obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+        stale = force or not _newer(obj, [src_path] + hdrs)
+        if only is not None and src not in only:
+            if not stale:
+                objs.append(obj)     # (built earlier and still current: stays in the library)
+            continue
         objs.append(obj)
-        if force or not _newer(obj, [src_path] + hdrs):
+        if stale:
             todo.append((src_path, obj))
 
     def compile_one(item):
@@ -86,7 +107,7 @@ def _build(hipcc, OBJ_DIR, LIB, extra, force, jobs, verbose, swap) -> str:
         return src_path
 
     if todo:
-        jobs = jobs or min(len(todo), os.cpu_count() or 4)
+        jobs = jobs or min(len(todo), os.cpu_count() or 4, 16)
         with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
             for done in ex.map(compile_one, todo):
                 if verbose:

@@ -1,0 +1,183 @@
+// moe.hip — mixture-of-experts feed-forward: fp32 router with top-k selection, and the expert products for the
+// token counts where an expert's weights are streamed once per assignment (decode and short portions).
+//
+//   swl_moe_route:        logits = router h + bias in fp32; the `top` largest (ties: lowest expert id); weights =
+//                         softmax over the chosen logits only.
+//   swl_moe_gate_up:      for every (token, chosen expert): g = min(W_gate h, limit), u = clamp(W_up h, +-limit),
+//                         y = g * sigmoid(1.702 g) * (u + 1); fp32 accumulation, y rounded to the compute dtype.
+//   swl_moe_down_combine: out[t] = sum_j weight[t][j] * (W_down[e_j] y[t][j]) with fp32 accumulation through the weighted
+//                         sum (fixed order j = 0, 1, ...: the result does not depend on what else is in the batch).
+//
+// Expert weights are stacked: gate_up [experts, 2 ff, width] (gate rows, then up rows), down [experts, width, ff].
+#include "swl_common.h"
+
+namespace swl {
+
+constexpr int kMoeThreads = 256;
+constexpr int kMoeWaves = kMoeThreads / 64;
+
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void moe_route_kernel(int32_t *idx_out, float *w_out, const T *h,
+                                                                const float *router, const float *bias, int width,
+                                                                int experts, int top) {
+    extern __shared__ float lds[];
+    float *hf = lds;                // [width]
+    float *logit = lds + width;     // [experts]
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int i = threadIdx.x; i < width; i += kMoeThreads) hf[i] = to_f(h[t * width + i]);
+    __syncthreads();
+    for (int e = wave; e < experts; e += kMoeWaves) {
+        const float *wr = router + static_cast<int64_t>(e) * width;
+        float a = 0.f;
+        for (int i = lane; i < width; i += 64) a += hf[i] * wr[i];
+        a = wave_allreduce_sum(a);
+        if (lane == 0) logit[e] = a + bias[e];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // top-k by repeated arg-max over the wave (each lane scans experts lane, lane + 64, ...)
+    float chosen_max = 0.f, denom = 0.f;
+    for (int j = 0; j < top; ++j) {
+        float best = -INFINITY;
+        int besti = 0x7fffffff;
+        for (int e = lane; e < experts; e += 64) {
+            const float v = logit[e];
+            if (v > best) {     // strict: keeps the lowest id among a lane's equals (NaN / taken entries never win)
+                best = v;
+                besti = e;
+            }
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) {
+            const float ob = __shfl_xor(best, m, 64);
+            const int oi = __shfl_xor(besti, m, 64);
+            if (ob > best || (ob == best && oi < besti)) {
+                best = ob;
+                besti = oi;
+            }
+        }
+        if (j == 0) chosen_max = best;
+        const float pj = expf(best - chosen_max);
+        denom += pj;
+        if (lane == 0) {
+            idx_out[t * top + j] = besti;
+            w_out[t * top + j] = pj;
+            logit[besti] = -INFINITY;
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+    if (lane == 0)
+        for (int j = 0; j < top; ++j) w_out[t * top + j] /= denom;
+}
+
+// grid (assignments, ceil(ff / 64)): wave w of the workgroup computes ff rows f0 + w, f0 + w + 4, ...
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void moe_gate_up_kernel(T *y, const T *h, const T *gate_up,
+                                                                  const int32_t *expert_idx, int width, int ff, int top,
+                                                                  float limit) {
+    extern __shared__ float lds[];
+    float *hf = lds;    // [width]
+    const int64_t a = blockIdx.x;           // assignment = token * top + j
+    const int64_t t = a / top;
+    const int e = expert_idx[a];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int i = threadIdx.x; i < width; i += kMoeThreads) hf[i] = to_f(h[t * width + i]);
+    __syncthreads();
+    const T *wg = gate_up + static_cast<int64_t>(e) * 2 * ff * width;
+    const T *wu = wg + static_cast<int64_t>(ff) * width;
+    const int f0 = blockIdx.y * 64;
+    for (int f = f0 + wave; f < min(ff, f0 + 64); f += kMoeWaves) {
+        const T *rg = wg + static_cast<int64_t>(f) * width, *ru = wu + static_cast<int64_t>(f) * width;
+        float g = 0.f, u = 0.f;
+        for (int i = lane; i < width; i += 64) {
+            const float x = hf[i];
+            g += x * to_f(rg[i]);
+            u += x * to_f(ru[i]);
+        }
+        g = wave_allreduce_sum(g);
+        u = wave_allreduce_sum(u);
+        if (lane == 0) {
+            g = fminf(g, limit);
+            u = fminf(fmaxf(u, -limit), limit);
+            const float sg = 1.0f / (1.0f + expf(-1.702f * g));
+            y[a * ff + f] = to_t<T>(g * sg * (u + 1.0f));
+        }
+    }
+}
+
+// grid (tokens, ceil(width / 64)): wave w computes output columns c0 + w, c0 + w + 4, ...
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void moe_down_combine_kernel(T *out, const T *y, const T *down,
+                                                                       const int32_t *expert_idx, const float *expert_w,
+                                                                       int width, int ff, int top) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c0 = blockIdx.y * 64;
+    for (int c = c0 + wave; c < min(width, c0 + 64); c += kMoeWaves) {
+        float total = 0.f;
+        for (int j = 0; j < top; ++j) {
+            const int e = expert_idx[t * top + j];
+            const T *wr = down + (static_cast<int64_t>(e) * width + c) * ff;
+            const T *yr = y + (t * top + j) * ff;
+            float a = 0.f;
+            for (int i = lane; i < ff; i += 64) a += to_f(yr[i]) * to_f(wr[i]);
+            a = wave_allreduce_sum(a);
+            total += expert_w[t * top + j] * a;
+        }
+        if (lane == 0) out[t * width + c] = to_t<T>(total);
+    }
+}
+
+} // namespace swl
+
+extern "C" int swl_moe_route(int32_t *idx_out, float *w_out, const void *h, const float *router, const float *bias,
+                             int64_t num_tokens, int32_t width, int32_t experts, int32_t top, int32_t dtype,
+                             swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || experts <= 0 || top <= 0 || top > experts) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!idx_out || !w_out || !h || !router || !bias) return SWL_ERR_BAD_ARG;
+    const size_t lds = (static_cast<size_t>(width) + experts) * 4;
+    if (num_tokens > 0x7fffffffLL || lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::moe_route_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kMoeThreads),
+                           lds, static_cast<hipStream_t>(stream), idx_out, w_out, static_cast<const T *>(h), router, bias,
+                           width, experts, top);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_moe_gate_up(void *y, const void *h, const void *gate_up, const int32_t *expert_idx,
+                               int64_t num_tokens, int32_t width, int32_t ff, int32_t top, float limit, int32_t dtype,
+                               swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || ff <= 0 || top <= 0) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!y || !h || !gate_up || !expert_idx) return SWL_ERR_BAD_ARG;
+    const size_t lds = static_cast<size_t>(width) * 4;
+    const int64_t assignments = num_tokens * top;
+    if (assignments > 0x7fffffffLL || lds > 64 * 1024 || (ff + 63) / 64 > 65535) return SWL_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(assignments), static_cast<unsigned>((ff + 63) / 64));
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::moe_gate_up_kernel<T>), grid, dim3(swl::kMoeThreads), lds,
+                           static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(h),
+                           static_cast<const T *>(gate_up), expert_idx, width, ff, top, limit);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_moe_down_combine(void *out, const void *y, const void *down, const int32_t *expert_idx,
+                                    const float *expert_w, int64_t num_tokens, int32_t width, int32_t ff, int32_t top,
+                                    int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || ff <= 0 || top <= 0) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!out || !y || !down || !expert_idx || !expert_w) return SWL_ERR_BAD_ARG;
+    if (num_tokens > 0x7fffffffLL || (width + 63) / 64 > 65535) return SWL_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(num_tokens), static_cast<unsigned>((width + 63) / 64));
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::moe_down_combine_kernel<T>), grid, dim3(swl::kMoeThreads), 0,
+                           static_cast<hipStream_t>(stream), static_cast<T *>(out), static_cast<const T *>(y),
+                           static_cast<const T *>(down), expert_idx, expert_w, width, ff, top);
+    });
+    return swl::check_launch();
+}

@@ -1,0 +1,81 @@
+// qknorm_kv.hip — per-head RMS norm of queries and keys fused with the paged KV store.
+//
+// One workgroup per token of the step (prompt portions and decoded tokens alike: every token carries its own sequence
+// row and position). The query heads are normalised in place inside the fused qkv projection output; the key heads are
+// normalised on their way into the K pool; the value heads are copied into the V pool. Norm statistics are fp32; the
+// norm weight is shared by all heads (plain weight, not one-plus).
+//
+// Pool layout: block b of a layer run's keys starts at k_cache + b * block_stride and holds [kv_heads, 16, dim]; its values
+// start at v_cache + b * block_stride and hold [kv_heads, 16, vdim] (block_stride in elements: a block of the pool may hold the
+// keys and values of several layer runs side by side, so that swapping moves one contiguous piece per block).
+#include "swl_common.h"
+
+namespace swl {
+
+constexpr int kQkThreads = 256;
+constexpr int kQkBlock = 16;    // tokens per KV block
+
+template <typename T>
+__global__ __launch_bounds__(kQkThreads) void qknorm_store_kv_kernel(
+    T *qkv, const float *q_w, const float *k_w, T *k_cache, T *v_cache, const int32_t *block_table,
+    const int32_t *tok_seq, const int32_t *tok_pos, int H, int G, int d, int dv, int64_t tok_stride,
+    int max_blocks_per_seq, int64_t block_stride, float eps, int store) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    T *row = qkv + t * tok_stride;
+    const int pos = tok_pos[t];
+    int64_t blk = 0;
+    if (store) blk = block_table[static_cast<int64_t>(tok_seq[t]) * max_blocks_per_seq + pos / kQkBlock];
+    const int off = pos % kQkBlock;
+    // heads 0..H-1: queries (in place); H..H+G-1: keys (into the pool)
+    for (int h = wave; h < H + G; h += kQkThreads / 64) {
+        const bool is_q = h < H;
+        const T *src = row + static_cast<int64_t>(h) * d;       // k heads follow the q heads: same formula
+        float ss = 0.f;
+        for (int e = lane; e < d; e += 64) {
+            const float v = to_f(src[e]);
+            ss += v * v;
+        }
+        ss = wave_allreduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+        if (is_q) {
+            T *dst = row + static_cast<int64_t>(h) * d;
+            for (int e = lane; e < d; e += 64) dst[e] = to_t<T>(to_f(src[e]) * r * q_w[e]);
+        } else if (store) {
+            const int g = h - H;
+            T *dst = k_cache + blk * block_stride + (static_cast<int64_t>(g) * kQkBlock + off) * d;
+            for (int e = lane; e < d; e += 64) dst[e] = to_t<T>(to_f(src[e]) * r * k_w[e]);
+        }
+    }
+    if (store) {
+        const T *vsrc = row + static_cast<int64_t>(H + G) * d;
+        for (int i = threadIdx.x; i < G * dv; i += kQkThreads) {
+            const int g = i / dv, c = i - g * dv;
+            v_cache[blk * block_stride + (static_cast<int64_t>(g) * kQkBlock + off) * dv + c] = vsrc[i];
+        }
+    }
+}
+
+} // namespace swl
+
+extern "C" int swl_qknorm_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_cache, void *v_cache,
+                                   const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                                   int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
+                                   int32_t vdim, int64_t tok_stride, int32_t max_blocks_per_seq, int64_t block_stride,
+                                   float eps, int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || dim <= 0 || vdim <= 0) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!qkv || !q_w || !k_w || !tok_pos) return SWL_ERR_BAD_ARG;
+    const int store = k_cache != nullptr;
+    if (store && (!v_cache || !block_table || !tok_seq)) return SWL_ERR_BAD_ARG;
+    if (tok_stride < static_cast<int64_t>(num_q_heads + num_kv_heads) * dim + static_cast<int64_t>(num_kv_heads) * vdim)
+        return SWL_ERR_BAD_ARG;
+    if (num_tokens > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::qknorm_store_kv_kernel<T>), dim3(static_cast<unsigned>(num_tokens)),
+                           dim3(swl::kQkThreads), 0, static_cast<hipStream_t>(stream), static_cast<T *>(qkv), q_w, k_w,
+                           static_cast<T *>(k_cache), static_cast<T *>(v_cache), block_table, tok_seq, tok_pos,
+                           num_q_heads, num_kv_heads, dim, vdim, tok_stride, max_blocks_per_seq, block_stride, eps, store);
+    });
+    return swl::check_launch();
+}

@@ -15,7 +15,8 @@ extern "C" int swl_swap_blocks(const int64_t *src_ids, const int64_t *dst_ids,
                                swl_stream_t stream) {
     if (num_blocks_to_swap < 0 || block_bytes <= 0) return SWL_ERR_BAD_ARG;
     if (num_blocks_to_swap == 0) return SWL_OK;
-    if (!src_ids || !dst_ids || !k_cache || !v_cache || !k_swap || !v_swap) return SWL_ERR_BAD_ARG;
+    if (!src_ids || !dst_ids || !k_cache || !k_swap || (v_cache == nullptr) != (v_swap == nullptr)) return SWL_ERR_BAD_ARG;
+    const bool two = v_cache != nullptr;    // (a model that keeps keys and values in one pool passes no second pair)
     hipStream_t s = static_cast<hipStream_t>(stream);
     char *kc = static_cast<char *>(k_cache), *vc = static_cast<char *>(v_cache);
     char *ks = static_cast<char *>(k_swap), *vs = static_cast<char *>(v_swap);
@@ -28,13 +29,13 @@ extern "C" int swl_swap_blocks(const int64_t *src_ids, const int64_t *dst_ids,
         const size_t bytes = static_cast<size_t>(run_end - run_begin) * block_bytes;
         const size_t src_off = static_cast<size_t>(src_ids[run_begin]) * block_bytes;
         const size_t dst_off = static_cast<size_t>(dst_ids[run_begin]) * block_bytes;
-        hipError_t e1, e2;
+        hipError_t e1, e2 = hipSuccess;
         if (is_swap_in) { // host swap pool -> GPU pool
             e1 = hipMemcpyAsync(kc + dst_off, ks + src_off, bytes, hipMemcpyHostToDevice, s);
-            e2 = hipMemcpyAsync(vc + dst_off, vs + src_off, bytes, hipMemcpyHostToDevice, s);
+            if (two) e2 = hipMemcpyAsync(vc + dst_off, vs + src_off, bytes, hipMemcpyHostToDevice, s);
         } else { // GPU pool -> host swap pool
             e1 = hipMemcpyAsync(ks + dst_off, kc + src_off, bytes, hipMemcpyDeviceToHost, s);
-            e2 = hipMemcpyAsync(vs + dst_off, vc + src_off, bytes, hipMemcpyDeviceToHost, s);
+            if (two) e2 = hipMemcpyAsync(vs + dst_off, vc + src_off, bytes, hipMemcpyDeviceToHost, s);
         }
         if (e1 != hipSuccess || e2 != hipSuccess) return SWL_ERR_RUNTIME;
         run_begin = run_end;

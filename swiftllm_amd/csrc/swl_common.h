@@ -283,3 +283,20 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
             return SWL_ERR_BAD_ARG;                  \
         }                                            \
     } while (0)
+
+// ... and the variant for operators that also run in true fp32 (SWL_F32).
+#define SWL_DISPATCH_DTYPE3(dtype, T, ...)           \
+    do {                                             \
+        if ((dtype) == SWL_F16) {                    \
+            using T = swl::f16;                      \
+            __VA_ARGS__                              \
+        } else if ((dtype) == SWL_BF16) {            \
+            using T = swl::bf16;                     \
+            __VA_ARGS__                              \
+        } else if ((dtype) == SWL_F32) {             \
+            using T = float;                         \
+            __VA_ARGS__                              \
+        } else {                                     \
+            return SWL_ERR_BAD_ARG;                  \
+        }                                            \
+    } while (0)

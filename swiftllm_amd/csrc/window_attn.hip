@@ -1,0 +1,175 @@
+// window_attn.hip — attention over the paged KV pool with a sliding window, tanh soft-capping and pre-softmax head
+// mixing ("talking heads": the capped scores of all query heads at one (query, key) pair are mixed by an [H, H] matrix
+// before the softmax), for any mixture of prompt portions and single decoded tokens.
+//
+// Every query token carries its sequence row and position; its own key/value are already in the pool (qknorm_kv.hip ran
+// first), so a prompt portion that continues a cached prefix, a whole prompt and a decoded token are the same case:
+// keys [max(0, p - window + 1), p] of the token's sequence, read through the block table.
+//
+// Because the mix couples the heads, one workgroup owns ALL heads of its query token. Keys are taken in chunks of 64:
+//   1. capped scores s[g][j] for every head g (fp32 dot products, fp32 tanh),
+//   2. mixed scores  m[h][j] = sum_g talk[h][g] s[g][j], online softmax per mixed head h (fp32, full-precision exp),
+//   3. acc[h][:] = acc[h][:] * alpha[h] + sum_j p[h][j] v[kv(h)][j][:]   (fp32 weights, fp32 accumulation).
+// This is the reference-grade kernel: everything after the loads is fp32 whatever the storage dtype.
+#include "swl_common.h"
+
+namespace swl {
+
+constexpr int kWaThreads = 256;
+constexpr int kWaChunk = 64;        // keys per chunk = one key per lane in the softmax phase
+constexpr int kWaBlock = 16;        // tokens per KV block
+constexpr int kWaMaxAcc = 32;       // (head, value column) accumulators per thread: H * vdim <= 8192
+
+// fp32 words ahead of the 8-byte-aligned key tables
+__host__ __device__ inline size_t wa_float_count(int H, int d) {
+    size_t n = static_cast<size_t>(H) * d + static_cast<size_t>(H) * H + 2 * static_cast<size_t>(H) * kWaChunk +
+               2 * static_cast<size_t>(H);
+    return n + (n & 1);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
+    T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
+    const int32_t *tok_pos, const float *talk, int H, int G, int d, int dv, int64_t q_tok_stride, int window,
+    float scale, float softcap, int max_blocks_per_seq, int64_t block_stride) {
+    extern __shared__ float lds[];
+    float *qf = lds;                        // [H * d]
+    float *tk = qf + H * d;                 // [H * H]
+    float *s = tk + H * H;                  // [H][64] capped scores
+    float *p = s + H * kWaChunk;            // [H][64] softmax numerators
+    float *alpha = p + H * kWaChunk;        // [H]
+    float *lsum = alpha + H;                // [H]
+    int64_t *kbase = reinterpret_cast<int64_t *>(lds + wa_float_count(H, d));   // [64] block id of each key (8-byte aligned)
+    int *koff = reinterpret_cast<int *>(kbase + kWaChunk);                          // [64] slot inside the block
+
+    const int64_t t = blockIdx.x;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int pos = tok_pos[t];
+    const int32_t *bt = block_table + static_cast<int64_t>(tok_seq[t]) * max_blocks_per_seq;
+    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int nkeys = pos - lo + 1;
+    const int rep = H / G;
+
+    const T *qrow = q + t * q_tok_stride;
+    for (int i = tid; i < H * d; i += kWaThreads) qf[i] = to_f(qrow[i]);
+    for (int i = tid; i < H * H; i += kWaThreads) tk[i] = talk[i];
+
+    float acc[kWaMaxAcc];
+#pragma unroll
+    for (int i = 0; i < kWaMaxAcc; ++i) acc[i] = 0.f;
+    // running maximum and sum of mixed head h live in the lanes of the wave that owns h (wave = h % 4): replicated
+    float mrun[8], lrun[8];     // heads per wave <= 8 -> H <= 32 ... generalised below through LDS when H > 32
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { mrun[i] = kNegBig; lrun[i] = 0.f; }
+    const int hpw = (H + 3) / 4;     // heads per wave (host guarantees <= 8)
+    const int nacc = (H * dv + kWaThreads - 1) / kWaThreads;
+
+    for (int c0 = 0; c0 < nkeys; c0 += kWaChunk) {
+        const int cn = min(kWaChunk, nkeys - c0);
+        __syncthreads();    // previous chunk's p / alpha / kbase fully consumed (and qf / tk written, first time)
+        if (tid < kWaChunk) {
+            const int kp = lo + c0 + tid;
+            if (tid < cn) {
+                kbase[tid] = bt[kp / kWaBlock];
+                koff[tid] = kp % kWaBlock;
+            }
+        }
+        __syncthreads();
+        // 1. capped scores
+        for (int idx = tid; idx < H * kWaChunk; idx += kWaThreads) {
+            const int g = idx / kWaChunk, j = idx - g * kWaChunk;
+            float v = 0.f;
+            if (j < cn) {
+                const T *kr = k_cache + kbase[j] * block_stride + (static_cast<int64_t>(g / rep) * kWaBlock + koff[j]) * d;
+                const float *qh = qf + g * d;
+                float a = 0.f;
+                for (int e = 0; e < d; ++e) a += qh[e] * to_f(kr[e]);
+                a *= scale;
+                v = softcap > 0.f ? softcap * tanhf(a / softcap) : a;
+            }
+            s[idx] = v;
+        }
+        __syncthreads();
+        // 2. mix the heads, online softmax per mixed head (wave `wave` owns heads wave, wave + 4, ...)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int h = wave + 4 * i;
+            if (i >= hpw || h >= H) break;
+            float mixed = kNegBig;
+            if (lane < cn) {
+                float a = 0.f;
+                for (int g = 0; g < H; ++g) a += tk[h * H + g] * s[g * kWaChunk + lane];
+                mixed = a;
+            }
+            const float cmax = wave_allreduce_max(mixed);
+            const float mnew = fmaxf(mrun[i], cmax);
+            const float pj = lane < cn ? expf(mixed - mnew) : 0.f;
+            const float csum = wave_allreduce_sum(pj);
+            const float al = expf(mrun[i] - mnew);      // first chunk: exp(-1e30 - m) = 0
+            lrun[i] = lrun[i] * al + csum;
+            mrun[i] = mnew;
+            p[h * kWaChunk + lane] = pj;
+            if (lane == 0) {
+                alpha[h] = al;
+                lsum[h] = lrun[i];
+            }
+        }
+        __syncthreads();
+        // 3. weighted values
+#pragma unroll
+        for (int i = 0; i < kWaMaxAcc; ++i) {
+            if (i >= nacc) break;
+            const int idx = tid + i * kWaThreads;
+            if (idx < H * dv) {
+                const int h = idx / dv, col = idx - h * dv;
+                const int g = h / rep;
+                float a = acc[i] * alpha[h];
+                const float *ph = p + h * kWaChunk;
+                for (int j = 0; j < cn; ++j) {
+                    const T *vr = v_cache + kbase[j] * block_stride + (static_cast<int64_t>(g) * kWaBlock + koff[j]) * dv;
+                    a += ph[j] * to_f(vr[col]);
+                }
+                acc[i] = a;
+            }
+        }
+    }
+    __syncthreads();
+    T *orow = out + t * static_cast<int64_t>(H) * dv;
+#pragma unroll
+    for (int i = 0; i < kWaMaxAcc; ++i) {
+        if (i >= nacc) break;
+        const int idx = tid + i * kWaThreads;
+        if (idx < H * dv) orow[idx] = to_t<T>(acc[i] / lsum[idx / dv]);
+    }
+}
+
+inline size_t wa_lds_bytes(int H, int d) {
+    return wa_float_count(H, d) * 4 + kWaChunk * (8 + 4);
+}
+
+} // namespace swl
+
+extern "C" int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v_cache,
+                               const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                               const float *talk, int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads,
+                               int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window, float scale,
+                               float softcap, int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
+                               swl_stream_t stream) {
+    if (num_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || dim <= 0 || vdim <= 0 || window < 0)
+        return SWL_ERR_BAD_ARG;
+    if (num_q_heads % num_kv_heads) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !talk) return SWL_ERR_BAD_ARG;
+    const size_t lds = swl::wa_lds_bytes(num_q_heads, dim);
+    if (num_tokens > 0x7fffffffLL || num_q_heads > 32 ||
+        static_cast<int64_t>(num_q_heads) * vdim > swl::kWaMaxAcc * swl::kWaThreads || lds > 64 * 1024)
+        return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::window_attn_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kWaThreads),
+                           lds, static_cast<hipStream_t>(stream), static_cast<T *>(out), static_cast<const T *>(q),
+                           static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, tok_seq,
+                           tok_pos, talk, num_q_heads, num_kv_heads, dim, vdim, q_tok_stride, window, scale, softcap,
+                           max_blocks_per_seq, block_stride);
+    });
+    return swl::check_launch();
+}

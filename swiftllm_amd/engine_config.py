@@ -36,6 +36,8 @@ class EngineConfig:
     # rounding points everywhere, so the bfloat16-only deferred norm (defer_rmsnorm, tiny_decode_batches) is off for it;
     # since r06c its row-owned projections run the EXACT norm on the fly instead (rows_decode: the same 5-6 launches per
     # layer with fused_add_rmsnorm's arithmetic — 3.95 vs 4.10 ms per step at batch 32, 3.11 vs 3.25 at batch 1).
+    # "float32" (true fp32 products, fp32 pool) is served by the models that list it in SUPPORTED_DTYPES (Kekapel); LLaMA's
+    # kernels are 16-bit only and its worker refuses it.
     dtype: str = "float16"
     # One [h + 2*KVH*D, h] GEMM instead of three (the reference left this commented out,
     # weight.py:131). fuse_qkv=False + use_skinny_gemm=False reproduces the reference's exact BLAS calls.
@@ -101,8 +103,8 @@ class EngineConfig:
             raise ValueError(
                 f"block_size={self.block_size} is not supported: the MI355X kernels are built for "
                 f"{self.SUPPORTED_BLOCK_SIZE}-token KV blocks (pass --block-size {self.SUPPORTED_BLOCK_SIZE})")
-        if self.dtype not in ("float16", "bfloat16"):
-            raise ValueError(f"dtype must be 'float16' or 'bfloat16', got {self.dtype!r}")
+        if self.dtype not in ("float16", "bfloat16", "float32"):
+            raise ValueError(f"dtype must be 'float16', 'bfloat16' or 'float32', got {self.dtype!r}")
         unknown = set(self.tuning or ()) - set(self.TUNING_DEFAULTS)
         if unknown:
             raise ValueError(f"unknown tuning switches {sorted(unknown)}; known: {sorted(self.TUNING_DEFAULTS)}")
@@ -130,7 +132,7 @@ class EngineConfig:
                        help="Sequences per forward, at most")
         g.add_argument("--max-tokens-in-batch", type=int, default=32768,
                        help="Tokens per forward, at most")
-        g.add_argument("--dtype", type=str, default="float16", choices=["float16", "bfloat16"])
+        g.add_argument("--dtype", type=str, default="float16", choices=["float16", "bfloat16", "float32"])
         g.add_argument("--no-fuse-qkv", dest="fuse_qkv", action="store_false")
         g.add_argument("--use-hip-graph", dest="use_hip_graph", action="store_true", default=True,
                        help="(default) replay captured hipGraphs for pure-decode steps")

@@ -38,3 +38,122 @@ class LlamaModelConfig:
     def load_from_model_path(model_path: str) -> "LlamaModelConfig":
         with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
             return LlamaModelConfig(json.load(f))
+
+
+class KekapelMixerConfig:
+    """Sizes and constants of one attention mixer (config `layers[i].mixer`)."""
+
+    def __init__(self, mixer: dict):
+        self.num_q_heads = int(mixer["heads"])
+        self.num_kv_heads = int(mixer.get("kv_heads", self.num_q_heads))
+        self.head_dim = int(mixer["dim"])
+        self.value_dim = int(mixer.get("vdim", self.head_dim))
+        self.scale = float(mixer["scale"])
+        cap = mixer.get("softcap")
+        self.softcap = float(cap) if cap else 0.0           # 0: scores are not capped
+        mask = mixer.get("mask") or {}
+        self.window = int(mask["size"]) if mask.get("size") else 0     # 0: every earlier key is visible
+        if self.num_q_heads % self.num_kv_heads:
+            raise ValueError(f"heads ({self.num_q_heads}) must be a multiple of kv_heads ({self.num_kv_heads})")
+
+    @property
+    def q_size(self) -> int:
+        return self.num_q_heads * self.head_dim
+
+    @property
+    def k_size(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def v_size(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+
+class KekapelMlpConfig:
+    """Feed-forward of one layer: `dense` (PolyNorm activation) or `moe` (router + clamped gated experts)."""
+
+    def __init__(self, mlp: dict):
+        self.kind = mlp["kind"]
+        if self.kind == "dense":
+            self.ffn_inter_dim = int(mlp["ff"])
+        elif self.kind == "moe":
+            self.ffn_inter_dim = int(mlp["expert"]["ff"])
+            self.limit = float(mlp["expert"]["limit"])
+            self.num_experts = int(mlp["router"]["experts"])
+            self.top_k = int(mlp["router"]["top"])
+            if not 0 < self.top_k <= self.num_experts:
+                raise ValueError(f"router.top ({self.top_k}) must be in 1..experts ({self.num_experts})")
+        else:
+            raise ValueError(f"unsupported mlp.kind {self.kind!r}")
+
+
+class KekapelLayerConfig:
+    def __init__(self, layer: dict):
+        if layer["type"] != "attention":
+            raise ValueError(f"unsupported layer type {layer['type']!r}")
+        self.type = layer["type"]
+        self.mixer = KekapelMixerConfig(layer["mixer"])
+        self.mlp = KekapelMlpConfig(layer["mlp"]) if layer.get("mlp") else None
+
+
+class LayerRun:
+    """One execution of a layer: `layer` indexes the weights, `index` the KV pool slice (a looped layer has one per pass),
+    `pass_index` >= 0 on the first layer of a loop pass (where the pass's step vector — and, after the first pass, the
+    embedding output — is added to the stream), else -1."""
+    __slots__ = ("index", "layer", "pass_index")
+
+    def __init__(self, index: int, layer: int, pass_index: int):
+        self.index, self.layer, self.pass_index = index, layer, pass_index
+
+
+class KekapelModelConfig:
+    """Kekapel: a decoder-only model with learned positions, sandwich LayerNorms around every sublayer, sliding-window
+    attention with q/k norm, tanh soft-capping and pre-softmax head mixing, dense (PolyNorm) or mixture-of-experts
+    feed-forwards, and a span of layers that runs several times with shared weights. Every size and constant is read from
+    config.json; layers may differ from one another."""
+
+    def __init__(self, model_config: dict):
+        if model_config.get("architecture") != "Kekapel":
+            raise AssertionError(f"unsupported architecture {model_config.get('architecture')!r}")
+        self.vocab_size = int(model_config["vocab"])
+        self.hidden_size = int(model_config["width"])
+        self.max_position_embeddings = int(model_config["max_positions"])
+        self.norm_eps = float(model_config["norm"]["eps"])
+        self.residual_mult = float(model_config.get("residual_mult", 1.0))
+        self.embedding_scale = float((model_config.get("embedding") or {}).get("scale", 1.0))
+        self.layers = [KekapelLayerConfig(layer) for layer in model_config["layers"]]
+        self.num_layers = len(self.layers)
+        loop = model_config.get("loop")
+        if loop:
+            self.loop_start, self.loop_stop, self.loop_times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
+            if not (0 <= self.loop_start < self.loop_stop <= self.num_layers and self.loop_times >= 1):
+                raise ValueError(f"bad loop {loop!r} for {self.num_layers} layers")
+        else:
+            self.loop_start = self.loop_stop = self.loop_times = 0
+        self.layer_runs = []
+        order = list(range(self.loop_start))
+        for t in range(self.loop_times):
+            order += [(i, t) for i in range(self.loop_start, self.loop_stop)]
+        order += list(range(self.loop_stop, self.num_layers))
+        for item in order:
+            layer, t = item if isinstance(item, tuple) else (item, -1)
+            first = t >= 0 and layer == self.loop_start
+            self.layer_runs.append(LayerRun(len(self.layer_runs), layer, t if first else -1))
+        self.num_layer_runs = len(self.layer_runs)
+        # what the scheduler-facing code reads off any model's configuration
+        self.num_q_heads = max(l.mixer.num_q_heads for l in self.layers)
+        self.num_kv_heads = max(l.mixer.num_kv_heads for l in self.layers)
+        self.head_dim = max(l.mixer.head_dim for l in self.layers)
+
+    def kv_elems_per_token(self) -> int:
+        """K and V elements one token occupies over all layer runs."""
+        return sum(self.layers[r.layer].mixer.k_size + self.layers[r.layer].mixer.v_size for r in self.layer_runs)
+
+    def get_kvslot_size(self, dtype: torch.dtype = torch.bfloat16) -> int:
+        """Bytes of KV cache one token occupies (every layer run has its own keys and values)."""
+        return self.kv_elems_per_token() * dtype.itemsize
+
+    @staticmethod
+    def load_from_model_path(model_path: str) -> "KekapelModelConfig":
+        with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
+            return KekapelModelConfig(json.load(f))

@@ -61,9 +61,9 @@ class Engine:
     async def initialize(self, num_gpu_blocks: Optional[int] = None):
         self.event_loop = asyncio.get_running_loop()
         if self.model is None:
-            from swiftllm_amd.worker.model import LlamaModel
+            from swiftllm_amd.registry import build_model
             print("[Engine] Initializing model...")
-            self.model = LlamaModel(self.engine_config)
+            self.model = build_model(self.engine_config)     # the worker class config.json's architecture names
             self.model_config = self.model.model_config
             print("[Engine] Loading weights...")
             self.model.load_weights()
@@ -81,6 +81,8 @@ class Engine:
         rope = getattr(self.model, "_cos_cached", None)
         if rope is not None:     # a request that would outgrow the rotary table is refused up front (HTTP 400),
             self.scheduler.max_seq_len = int(rope.shape[0])     # not left to raise inside forward mid-flight
+        elif getattr(self.model, "max_seq_len", None):          # (a model with a learned position table says so itself)
+            self.scheduler.max_seq_len = int(self.model.max_seq_len)
         self.tokenization_engine = TokenizationEngine(self.engine_config)
         if hasattr(self.model, "after_launch_hook"):
             self.model.after_launch_hook = self._post_undelivered

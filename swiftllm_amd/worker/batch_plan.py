@@ -132,3 +132,78 @@ def plan_batch(input_ids_list: Sequence[Sequence[int]], seq_ids_list: Sequence[i
         seq_lengths=np.asarray(seq_lengths_list, dtype=np.int32), prefill_seq_lens=pl,
         prefill_start_locs_with_end=starts_with_end, decoding_seq_lens=dl, position_indices=pos,
         last_token_indices=last)
+
+
+# ---- token-level steps: prompt portions and decoded tokens in one batch ----------------------------------------------------
+@dataclasses.dataclass
+class StepEntry:
+    """The tokens one sequence brings to a step: `tokens` continue the sequence at position `start` (0 for a new sequence;
+    a decoded token is a portion of length one). `want`: offsets inside `tokens` whose logits the caller asks for."""
+    seq_id: int
+    tokens: Sequence[int]
+    start: int
+    want: Sequence[int] = ()
+
+
+@dataclasses.dataclass
+class StepPlan:
+    """Flat per-token metadata of a step. Kernels that serve portions and decoded tokens alike need nothing else: a token's
+    block-table row, its position, and (for the output) which rows are asked for."""
+    num_tokens: int
+    num_seqs: int
+    seq_ids_list: List[int]
+    target_lens_list: List[int]         # length of every sequence after the step (what the block allocator must cover)
+    input_ids: np.ndarray               # [T] int32
+    tok_pos: np.ndarray                 # [T] int32 position of each token in its sequence
+    tok_seq: np.ndarray                 # [T] int32 block-table row of each token
+    want_rows: np.ndarray               # [R] int32 rows (into the T tokens) whose logits are produced
+
+    SEGMENTS = ("input_ids", "tok_pos", "tok_seq", "want_rows")
+
+    def packed_layout(self):
+        out, off = [], 0
+        for name in self.SEGMENTS:
+            n = getattr(self, name).size
+            out.append((name, off, n))
+            off += (n + 3) // 4 * 4
+        return out, off
+
+    def pack_into(self, buf: np.ndarray) -> int:
+        layout, total = self.packed_layout()
+        for name, off, n in layout:
+            buf[off:off + n] = getattr(self, name)
+        return total
+
+
+def plan_step(entries: Sequence[StepEntry], vocab_size: int = None, max_positions: int = None) -> StepPlan:
+    """Flatten the entries in order. Checked here, on the host, so that nothing out of range reaches a kernel: token ids
+    against the vocabulary, positions against the position table, one entry per sequence."""
+    ids, pos, seq, want, seq_ids, targets = [], [], [], [], [], []
+    base = 0
+    for e in entries:
+        n = len(e.tokens)
+        if n == 0:
+            raise ValueError(f"sequence {e.seq_id} brings no tokens to the step")
+        if e.start < 0:
+            raise ValueError(f"sequence {e.seq_id}: negative start {e.start}")
+        if max_positions is not None and e.start + n > max_positions:
+            raise RuntimeError(f"sequence {e.seq_id} would reach position {e.start + n - 1}, the model has "
+                               f"{max_positions} positions")
+        if e.seq_id in seq_ids:
+            raise ValueError(f"sequence {e.seq_id} appears twice in one step")
+        toks = np.asarray(e.tokens, dtype=np.int64)
+        if vocab_size is not None and (toks.min() < 0 or toks.max() >= vocab_size):
+            raise ValueError(f"sequence {e.seq_id}: token ids must be in [0, {vocab_size})")
+        ids.append(toks.astype(np.int32))
+        pos.append(np.arange(e.start, e.start + n, dtype=np.int32))
+        seq.append(np.full(n, e.seq_id, dtype=np.int32))
+        for w in e.want:
+            if not 0 <= w < n:
+                raise ValueError(f"sequence {e.seq_id}: wanted offset {w} outside its {n} tokens")
+            want.append(base + w)
+        seq_ids.append(int(e.seq_id))
+        targets.append(int(e.start + n))
+        base += n
+    cat = (lambda xs: np.concatenate(xs) if xs else np.empty(0, dtype=np.int32))
+    return StepPlan(num_tokens=base, num_seqs=len(seq_ids), seq_ids_list=seq_ids, target_lens_list=targets,
+                    input_ids=cat(ids), tok_pos=cat(pos), tok_seq=cat(seq), want_rows=np.asarray(want, dtype=np.int32))

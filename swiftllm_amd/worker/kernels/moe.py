@@ -1,0 +1,38 @@
+"""Mixture-of-experts feed-forward: fp32 router + top-k + softmax over the chosen logits, clamped gated experts, weighted
+combination. csrc/moe.hip."""
+import torch
+
+from swiftllm_amd import _hip
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top_k: int):
+    """-> (expert ids int32 [T, top_k], weights fp32 [T, top_k])."""
+    _hip.require_gpu_tensor(h, "h")
+    n, width = h.shape
+    experts = router.shape[0]
+    assert h.is_contiguous() and router.dtype == bias.dtype == torch.float32 and router.is_contiguous()
+    assert router.shape[1] == width and bias.numel() == experts
+    idx = torch.empty((n, top_k), dtype=torch.int32, device=h.device)
+    wts = torch.empty((n, top_k), dtype=torch.float32, device=h.device)
+    _hip.call("swl_moe_route", _hip.ptr(idx), _hip.ptr(wts), _hip.ptr(h), _hip.ptr(router), _hip.ptr(bias), n, width,
+              experts, top_k, _hip.dtype_code3(h.dtype), _hip.stream())
+    return idx, wts
+
+
+def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
+                limit: float) -> torch.Tensor:
+    """-> [T, width]: sum_j wts[t, j] * expert idx[t, j] applied to h[t]. gate_up [experts, 2 ff, width], down
+    [experts, width, ff]."""
+    n, width = h.shape
+    experts, two_ff, _ = gate_up.shape
+    ff, top_k = two_ff // 2, idx.shape[1]
+    assert gate_up.is_contiguous() and down.is_contiguous() and down.shape == (experts, width, ff)
+    assert gate_up.dtype == down.dtype == h.dtype and idx.dtype == torch.int32 and wts.dtype == torch.float32
+    code, stream = _hip.dtype_code3(h.dtype), _hip.stream()
+    y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
+    _hip.call("swl_moe_gate_up", _hip.ptr(y), _hip.ptr(h), _hip.ptr(gate_up), _hip.ptr(idx), n, width, ff, top_k,
+              float(limit), code, stream)
+    out = torch.empty((n, width), dtype=h.dtype, device=h.device)
+    _hip.call("swl_moe_down_combine", _hip.ptr(out), _hip.ptr(y), _hip.ptr(down), _hip.ptr(idx), _hip.ptr(wts), n, width,
+              ff, top_k, code, stream)
+    return out

@@ -1,0 +1,57 @@
+"""Attention over the paged pool for models whose heads are coupled before the softmax: per-head q/k RMS norm fused with
+the KV store, then sliding-window attention with tanh soft-capping and an [H, H] head-mixing matrix. Prompt portions (with
+or without a cached prefix) and decoded tokens go through the same two launches: every token carries its block-table row
+and its position. csrc/qknorm_kv.hip, csrc/window_attn.hip."""
+import torch
+
+from swiftllm_amd import _hip
+
+
+class PoolSlice:
+    """Where one layer run keeps its keys and values inside the shared block pool: element offsets inside a block."""
+    __slots__ = ("k_offset", "v_offset")
+
+    def __init__(self, k_offset: int, v_offset: int):
+        self.k_offset, self.v_offset = k_offset, v_offset
+
+
+def qknorm_and_store_kv(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: torch.Tensor, pool: torch.Tensor,
+                        pool_slice: PoolSlice, block_table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor,
+                        mixer, eps: float):
+    """qkv [T, q | k | v] of one fused projection: q heads normalised in place, k heads normalised into the pool, v heads
+    copied into the pool. pool None (memory profiling): only the query norm."""
+    _hip.require_gpu_tensor(qkv, "qkv")
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == mixer.q_size + mixer.k_size + mixer.v_size
+    assert q_norm.dtype == k_norm.dtype == torch.float32 and q_norm.numel() == k_norm.numel() == mixer.head_dim
+    assert tok_pos.dtype == torch.int32 and tok_pos.shape[0] == qkv.shape[0]
+    kp = vp = 0
+    stride = 0
+    if pool is not None:
+        assert pool.is_contiguous() and pool.dtype == qkv.dtype and block_table.is_contiguous()
+        assert tok_seq.dtype == torch.int32 and tok_seq.shape[0] == qkv.shape[0]
+        esize = pool.element_size()
+        kp = pool.data_ptr() + pool_slice.k_offset * esize
+        vp = pool.data_ptr() + pool_slice.v_offset * esize
+        stride = pool.shape[1]
+    _hip.call("swl_qknorm_store_kv", _hip.ptr(qkv), _hip.ptr(q_norm), _hip.ptr(k_norm), kp, vp, _hip.ptr(block_table),
+              _hip.ptr(tok_seq), _hip.ptr(tok_pos), qkv.shape[0], mixer.num_q_heads, mixer.num_kv_heads, mixer.head_dim,
+              mixer.value_dim, qkv.stride(0), block_table.shape[1] if block_table is not None else 0, stride, float(eps),
+              _hip.dtype_code3(qkv.dtype), _hip.stream())
+
+
+def window_attention(qkv: torch.Tensor, talk: torch.Tensor, pool: torch.Tensor, pool_slice: PoolSlice,
+                     block_table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, mixer) -> torch.Tensor:
+    """-> [T, heads * vdim]. The queries are the (already normalised) first columns of qkv; keys and values come from the
+    pool, which already holds this step's tokens."""
+    _hip.require_gpu_tensor(qkv, "qkv")
+    assert talk.dtype == torch.float32 and talk.is_contiguous() and talk.shape == (mixer.num_q_heads, mixer.num_q_heads)
+    assert pool.is_contiguous() and pool.dtype == qkv.dtype
+    n = qkv.shape[0]
+    out = torch.empty((n, mixer.num_q_heads * mixer.value_dim), dtype=qkv.dtype, device=qkv.device)
+    esize = pool.element_size()
+    _hip.call("swl_window_attn", _hip.ptr(out), _hip.ptr(qkv), pool.data_ptr() + pool_slice.k_offset * esize,
+              pool.data_ptr() + pool_slice.v_offset * esize, _hip.ptr(block_table), _hip.ptr(tok_seq), _hip.ptr(tok_pos),
+              _hip.ptr(talk), n, mixer.num_q_heads, mixer.num_kv_heads, mixer.head_dim, mixer.value_dim, qkv.stride(0),
+              mixer.window, float(mixer.scale), float(mixer.softcap), block_table.shape[1], pool.shape[1],
+              _hip.dtype_code3(qkv.dtype), _hip.stream())
+    return out

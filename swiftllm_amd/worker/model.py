@@ -72,6 +72,8 @@ class LlamaModel:
     def __init__(self, engine_config: EngineConfig):
         self.engine_config = engine_config
         self.model_config = LlamaModelConfig.load_from_model_path(engine_config.model_path)
+        if getattr(engine_config, "dtype", "float16") not in _DTYPES:
+            raise ValueError(f"LlamaModel runs in float16 or bfloat16, not {engine_config.dtype!r}")
         self.dtype = _DTYPES[getattr(engine_config, "dtype", "float16")]
         self.device = torch.device("cuda")
 
