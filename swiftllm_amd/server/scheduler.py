@@ -81,7 +81,7 @@ class Scheduler:
                 return f"prompt_token_ids must be integers in [0, {self.vocab_size})"
         if self.max_seq_len is not None and req.prompt_len + req.output_len > self.max_seq_len:
             return (f"prompt ({req.prompt_len}) + output_len ({req.output_len}) exceeds the model's "
-                    f"{self.max_seq_len} positions")
+                    f"{self.max_seq_len} positions (rotary table or learned position table)")
         if req.prompt_len > ecfg.max_tokens_in_batch:
             return f"prompt of {req.prompt_len} tokens exceeds max_tokens_in_batch ({ecfg.max_tokens_in_batch})"
         blocks = cdiv(req.prompt_len + req.output_len, ecfg.block_size)

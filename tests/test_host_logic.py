@@ -349,7 +349,9 @@ def test_engine_config_rejects_unsupported_block_size():
     with pytest.raises(ValueError, match="block_size=32"):
         EngineConfig(block_size=32, **base)
     with pytest.raises(ValueError, match="dtype"):
-        EngineConfig(block_size=16, dtype="float32", **base)
+        EngineConfig(block_size=16, dtype="float64", **base)
+    # true fp32 is an engine dtype (the models that serve it say so); LLaMA's 16-bit kernels refuse it in the worker
+    assert EngineConfig(block_size=16, dtype="float32", **base).dtype == "float32"
 
 
 def test_graph_bucket_keeps_splits_balanced_and_few():
