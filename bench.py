@@ -94,7 +94,112 @@ def parse_args():
     ap.add_argument("--kv-placement", default="top", choices=["top", "bottom"],
                     help="top: filler sequences occupy the low block ids, the run's sequences get the highest ones")
     ap.add_argument("--no-reference", action="store_true", help="skip the reference-Triton child run")
+    ap.add_argument("--compare-designs", action="store_true",
+                    help="instead of the headline workload: prefill and decode throughput of Kekapel beside LLaMA at equal "
+                         "layer sizes (random weights), one JSON line with both")
+    ap.add_argument("--compare-sizes", default="small,medium", help="comma list out of " + ",".join(COMPARE_SIZES))
     return ap.parse_args()
+
+
+# --compare-designs: layer sizes that resemble real models' (width, heads x head size, feed-forward width); both designs get
+# the same ones. Kekapel alternates dense and mixture-of-experts layers (experts of ff / 4, top 2 of 8: the active expert
+# width is half the dense one), windows of 1024 tokens, no loop (a loop re-runs layers: the per-layer cost is what is compared).
+COMPARE_SIZES = {
+    "small": dict(width=1024, layers=8, heads=8, kv_heads=2, dim=128, ff=4096, vocab=32000),
+    "medium": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, ff=8192, vocab=32000),
+    "wide": dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, ff=14336, vocab=32000),
+}
+
+
+def _compare_configs(sz, positions):
+    llama = dict(model_type="llama", hidden_act="silu", rms_norm_eps=1e-5, rope_scaling=None, tie_word_embeddings=False,
+                 num_hidden_layers=sz["layers"], hidden_size=sz["heads"] * sz["dim"], num_attention_heads=sz["heads"],
+                 num_key_value_heads=sz["kv_heads"], intermediate_size=sz["ff"], vocab_size=sz["vocab"],
+                 max_position_embeddings=positions, rope_theta=10000.0)
+    mixer = dict(dim=sz["dim"], vdim=sz["dim"], heads=sz["heads"], kv_heads=sz["kv_heads"], mask=dict(size=1024),
+                 scale=sz["dim"] ** -0.5, softcap=30.0)
+    dense = dict(kind="dense", ff=sz["ff"])
+    moe = dict(kind="moe", expert=dict(ff=sz["ff"] // 4, limit=7.0), router=dict(experts=8, top=2))
+    layers = [dict(type="attention", mixer=mixer, mlp=(moe if i % 2 else dense)) for i in range(sz["layers"])]
+    kekapel = dict(architecture="Kekapel", embedding=dict(scale=1.0), layers=layers, max_positions=positions,
+                   norm=dict(eps=1e-6), residual_mult=0.5, vocab=sz["vocab"], width=sz["width"])
+    return llama, kekapel
+
+
+def _compare_one(cfg, dtype, prompt_len, prompt_batch, decode_batch, decode_ctx, steps, warmup):
+    """Prefill tokens/s (prompt_batch whole prompts in one forward) and decode tokens/s (decode_batch sequences at context
+    decode_ctx, one token each per forward) of one design through its worker's forward()."""
+    import tempfile
+    import torch
+    from oracle import synth
+    from swiftllm_amd import EngineConfig, build_model
+    path = synth.write_model_dir(tempfile.mkdtemp(prefix="swl_cmp_"), cfg)
+    blocks = (prompt_batch * (prompt_len + 16) + decode_batch * (decode_ctx + steps + warmup + 32)) // 16 + 64
+    ecfg = EngineConfig(model_path=path, use_dummy=True, block_size=16, gpu_mem_utilization=0.9, num_cpu_blocks=0,
+                        max_seqs_in_block_table=max(prompt_batch, decode_batch) + 1,
+                        max_blocks_per_seq=(max(prompt_len, decode_ctx) + steps + warmup + 64) // 16 + 1,
+                        max_batch_size=max(prompt_batch, decode_batch), max_tokens_in_batch=prompt_batch * prompt_len,
+                        dtype=dtype, use_hip_graph=True)
+    model = build_model(ecfg)
+    model.load_weights()
+    model.init_kvcache_and_swap(blocks)
+    vocab = model.model_config.vocab_size
+    g = torch.Generator().manual_seed(0)
+    out = {}
+    prompts = [torch.randint(0, vocab, (prompt_len,), generator=g).tolist() for _ in range(prompt_batch)]
+    ids = list(range(prompt_batch))
+    times = []
+    for i in range(3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.forward(prompts, ids, [])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        model.free_seqs_resources(ids)
+    out["prefill_tokens_per_s"] = prompt_batch * prompt_len / min(times[1:])
+    out["prefill_ms"] = min(times[1:]) * 1e3
+    # decode: contexts come from one prefill of decode_ctx tokens per sequence (in slices that fit the token budget)
+    ids = list(range(decode_batch))
+    per = max(1, ecfg.max_tokens_in_batch // decode_ctx)
+    toks = [0] * decode_batch
+    for a in range(0, decode_batch, per):
+        chunk = ids[a:a + per]
+        res = model.forward([torch.randint(0, vocab, (decode_ctx,), generator=g).tolist() for _ in chunk], chunk, [])
+        toks[a:a + len(chunk)] = res
+    lens = [decode_ctx] * decode_batch
+    for i in range(warmup + steps):
+        if i == warmup:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+        lens = [n + 1 for n in lens]
+        toks = model.forward([[t] for t in toks], ids, lens)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    out["decode_tokens_per_s"] = decode_batch * steps / dt
+    out["decode_ms_per_step"] = dt / steps * 1e3
+    model.free_seqs_resources(ids)
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_compare_designs(args):
+    """Both designs at every requested size -> one JSON-able dict (rates in tokens/s; ratio = Kekapel / LLaMA)."""
+    results = {}
+    for name in [s for s in args.compare_sizes.split(",") if s]:
+        sz = COMPARE_SIZES[name]
+        prompt_len, prompt_batch, decode_batch, decode_ctx = 2048, 4, 32, 1024
+        llama, kekapel = _compare_configs(sz, prompt_len + 256)
+        rec = {"sizes": sz, "prompt": [prompt_batch, prompt_len], "decode": [decode_batch, decode_ctx]}
+        for label, cfg in (("llama", llama), ("kekapel", kekapel)):
+            rec[label] = _compare_one(cfg, args.dtype, prompt_len, prompt_batch, decode_batch, decode_ctx,
+                                      min(args.steps, 32), min(args.warmup, 8))
+            print(f"[compare] {name} {label}: {rec[label]}", file=sys.stderr, flush=True)
+        rec["prefill_ratio"] = rec["kekapel"]["prefill_tokens_per_s"] / rec["llama"]["prefill_tokens_per_s"]
+        rec["decode_ratio"] = rec["kekapel"]["decode_tokens_per_s"] / rec["llama"]["decode_tokens_per_s"]
+        results[name] = rec
+    return {"metric": "design_comparison_tokens_per_s", "dtype": args.dtype, "data": "synthetic", "n_gpus": 1,
+            "results": results}
 
 
 MODEL_DIMS = {
@@ -714,7 +819,7 @@ def main():
     os.dup2(2, 1)
     try:
         with contextlib.redirect_stdout(sys.stderr):
-            result = _run(args)
+            result = run_compare_designs(args) if args.compare_designs else _run(args)
     finally:
         sys.stdout.flush()
         os.dup2(saved, 1)

@@ -527,6 +527,18 @@ int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v
                     int32_t window, float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride,
                     int32_t dtype, swl_stream_t stream);
 
+/* The matrix-core form for 16-bit dtypes and head sizes 64 / 128: the step's tokens come as tiles of up to 16 consecutive
+ * tokens of one sequence (tile_row0[i] = first token row, tile_cnt[i] = tokens; a decoded token is a tile of one). Same
+ * arithmetic as swl_window_attn up to rounding (fp32 scores and weights; weights enter the value product as hi + lo 16-bit
+ * terms). swl_window_attn_tiles_supported: 1 when it serves the shape. */
+int swl_window_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int32_t dtype);
+int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
+                          const int32_t *tok_seq, const int32_t *tok_pos, const int32_t *tile_row0,
+                          const int32_t *tile_cnt, const float *talk, int32_t num_tiles, int32_t num_q_heads,
+                          int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window,
+                          float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
+                          swl_stream_t stream);
+
 /* ---- PolyNorm activation: out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row ---------- */
 int swl_polynorm(void *out, const void *z, float a, float b, float c, float e, float eps, int64_t num_rows, int32_t ff,
                  int32_t dtype, swl_stream_t stream);

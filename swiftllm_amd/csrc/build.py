@@ -32,6 +32,7 @@ SOURCES = [
     "layernorm.hip",
     "qknorm_kv.hip",
     "window_attn.hip",
+    "window_attn_mfma.hip",
     "polynorm.hip",
     "moe.hip",
 ]
@@ -41,7 +42,8 @@ SOURCES = [
 _SHARED = ["swap_blocks.hip", "block_table.hip", "argmax.hip", "gemm_skinny.hip", "gemm_wide.hip"]
 MODEL_SOURCES = {
     "llama": list(SOURCES[:14]),
-    "Kekapel": _SHARED + ["layernorm.hip", "qknorm_kv.hip", "window_attn.hip", "polynorm.hip", "moe.hip"],
+    "Kekapel": _SHARED + ["layernorm.hip", "qknorm_kv.hip", "window_attn.hip", "window_attn_mfma.hip",
+                          "polynorm.hip", "moe.hip"],
 }
 HEADERS = ["swl_common.h", "attend_block.h", os.path.join(ROOT, "include", "swiftllm_hip.h")]
 LIB = os.path.join(HERE, "libswiftllm_hip.so")

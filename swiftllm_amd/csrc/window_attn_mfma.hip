@@ -1,0 +1,280 @@
+// window_attn_mfma.hip — the matrix-core form of window_attn.hip for 16-bit storage: tiles of up to 16 consecutive query
+// tokens of one sequence against 16-key pages of the pool.
+//
+// One workgroup (4 waves) per query tile. The head mix couples all heads of a (query, key) pair, so the heads are split
+// over the waves: wave w owns heads [w * HPW, (w + 1) * HPW) for the score products AND for the outputs, and the capped
+// scores of all heads meet in LDS in between. Per 16-key page:
+//   1. S^T_g = K_kv(g) Q_g^T      (16 keys x 16 queries, MFMA 16x16x16, fp32 accumulate), scale, tanh cap -> LDS [H][256] fp32
+//   2. mixed_h = sum_g talk[h][g] S^T_g   (fp32 VALU, talk from scalar loads), window mask, online softmax per (h, query)
+//   3. O^T_h += V^T_kv(h) P^T_h   with the fp32 weights split into two 16-bit terms (hi + lo): the product keeps ~16 bits of
+//      every weight although the matrix core takes 16-bit operands.
+// The transposed products keep the query index on the lanes' low four bits in every stage, so the softmax statistics of a
+// query never move between lanes. Keys outside [pos - window + 1, pos] get weight zero; pages wholly outside are skipped.
+#include "swl_common.h"
+
+namespace swl {
+
+constexpr int kWmThreads = 256;
+constexpr int kWmWaves = 4;
+constexpr int kWmTile = 16;     // queries per tile = keys per page = MFMA edge
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+// D[16x16] += A[16x16] B[16x16]; lane l holds A[l % 16][4 (l / 16) + 0..3], B[4 (l / 16) + 0..3][l % 16], D[4 (l / 16) + 0..3][l % 16]
+__device__ __forceinline__ float4_t mfma16(const bf16 (&a)[4], const bf16 (&b)[4], float4_t c) {
+    short4v av, bv;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        av[i] = __builtin_bit_cast(short, a[i]);
+        bv[i] = __builtin_bit_cast(short, b[i]);
+    }
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av, bv, c, 0, 0, 0);
+}
+__device__ __forceinline__ float4_t mfma16(const f16 (&a)[4], const f16 (&b)[4], float4_t c) {
+    half4v av, bv;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        av[i] = a[i];
+        bv[i] = b[i];
+    }
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(av, bv, c, 0, 0, 0);
+}
+
+template <typename T>
+__device__ __forceinline__ void load4(T (&dst)[4], const T *p) {    // 8-byte load
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    const vec4 v = *reinterpret_cast<const vec4 *>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = v[i];
+}
+
+__device__ __forceinline__ float fast_tanh(float x) {
+    // 1 - 2 / (e^{2x} + 1); exp2 overflow to inf gives exactly 1, underflow to 0 gives exactly -1
+    const float e = fast_exp2(x * 2.885390081777927f);
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
+template <typename T, int D, int DV, int HPW>
+__global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
+    T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
+    const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk, int H, int G,
+    int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride) {
+    extern __shared__ float s_lds[];    // [H][64 lanes][4]
+    constexpr int CT = DV / 16;         // 16-column tiles of the value head
+    constexpr float kLog2e = 1.4426950408889634f;
+    const int tile = blockIdx.x;
+    const int row0 = tile_row0[tile], cnt = tile_cnt[tile];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int li = lane & 15, lq = lane >> 4;       // query (or operand row) index; quarter
+    const int p0 = tok_pos[row0];
+    const int32_t *bt = block_table + static_cast<int64_t>(tok_seq[row0]) * max_blocks_per_seq;
+    const int rep = H / G;
+    const int h0 = wave * HPW;
+    const int qpos = p0 + li;                        // this lane's query position (meaningful when li < cnt)
+    const bool qok = li < cnt;
+    const int lo_first = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+    const int kb0 = lo_first / kWmTile, kb1 = (p0 + cnt - 1) / kWmTile;
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+
+    float4_t acc[HPW][CT];
+    float mrun[HPW], lrun[HPW];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        mrun[hh] = kNegBig;
+        lrun[hh] = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc[hh][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    // the query row this lane feeds as B operand of S^T = K Q^T: row li of the tile (rows past cnt: the tile's last row)
+    const T *qrow = q + static_cast<int64_t>(row0 + (qok ? li : cnt - 1)) * q_tok_stride;
+
+    for (int kb = kb0; kb <= kb1; ++kb) {
+        const int64_t blk = bt[kb];
+        const T *kblk = k_cache + blk * block_stride;
+        const T *vblk = v_cache + blk * block_stride;
+        // ---- 1. capped scores of this wave's heads -> LDS -------------------------------------------------------------------
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+            const int g = h0 + hh;
+            if (g < H) {
+                const T *kr = kblk + (static_cast<int64_t>(g / rep) * kWmTile + li) * D + 4 * lq;   // A: key li, dims 4 lq ..
+                const T *qr = qrow + g * D + 4 * lq;                                                   // B: query li
+                float4_t st = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int e = 0; e < D; e += 16) {
+                    T a[4], b[4];
+                    load4(a, kr + e);
+                    load4(b, qr + e);
+                    st = mfma16(a, b, st);
+                }
+                mfma_results_ready<4>(st);
+                // st[r] = S^T[key 4 lq + r][query li]
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = st[r] * scale;
+                    if (softcap > 0.f) v = softcap * fast_tanh(v * inv_cap);
+                    st[r] = v;
+                }
+                *reinterpret_cast<float4_t *>(&s_lds[(g * 64 + lane) * 4]) = st;
+            }
+        }
+        __syncthreads();
+        // ---- 2. mix, mask, online softmax; 3. O^T += V^T P^T for this wave's heads ------------------------------------------
+        const int kpos0 = kb * kWmTile + 4 * lq;     // position of this lane's key r = 0
+        bool ok[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int kp = kpos0 + r;
+            ok[r] = qok && kp <= qpos && (window <= 0 || kp > qpos - window);
+        }
+        float mixed[HPW][4];
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mixed[hh][r] = 0.f;
+        for (int g = 0; g < H; ++g) {
+            const float4_t sv = *reinterpret_cast<const float4_t *>(&s_lds[(g * 64 + lane) * 4]);
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int h = min(h0 + hh, H - 1);
+                const float tw = talk[h * H + g];       // wave-uniform address: a scalar load
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mixed[hh][r] += tw * sv[r];
+            }
+        }
+        int prev_kv = -1;
+        T vfrag[CT][4];
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+            const int h = h0 + hh;
+            if (h < H) {
+                float cmax = kNegBig;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) cmax = fmaxf(cmax, ok[r] ? mixed[hh][r] : kNegBig);
+                cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+                cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+                const float mnew = fmaxf(mrun[hh], cmax);
+                const float alpha = fast_exp2((mrun[hh] - mnew) * kLog2e);
+                mrun[hh] = mnew;
+                T phi[4], plo[4];
+                float psum = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float pv = ok[r] ? fast_exp2((mixed[hh][r] - mnew) * kLog2e) : 0.f;
+                    psum += pv;
+                    phi[r] = to_t<T>(pv);
+                    plo[r] = to_t<T>(pv - to_f(phi[r]));
+                }
+                lrun[hh] = lrun[hh] * alpha + psum;
+                const int kv = h / rep;
+                if (kv != prev_kv) {    // (wave-uniform) A operand: V^T[col ct * 16 + li][key 4 lq + r]
+                    prev_kv = kv;
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            vfrag[ct][r] = vblk[(static_cast<int64_t>(kv) * kWmTile + 4 * lq + r) * DV + ct * 16 + li];
+                }
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    float4_t o = acc[hh][ct];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[r] *= alpha;
+                    o = mfma16(vfrag[ct], phi, o);
+                    o = mfma16(vfrag[ct], plo, o);
+                    acc[hh][ct] = o;
+                }
+            }
+        }
+        __syncthreads();    // every wave is done with this page's scores before the next page overwrites them
+    }
+    // ---- epilogue: O[query li][h][ct * 16 + 4 lq + r] = O^T / l -------------------------------------------------------------------
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        const int h = h0 + hh;
+        if (h < H) {
+            float l = lrun[hh];
+            l += __shfl_xor(l, 16, 64);
+            l += __shfl_xor(l, 32, 64);
+            const float inv = 1.0f / l;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                float4_t o = acc[hh][ct];
+                mfma_results_ready<4>(o);
+                if (qok) {
+                    typedef T vec4 __attribute__((ext_vector_type(4)));
+                    vec4 w;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) w[r] = to_t<T>(o[r] * inv);
+                    *reinterpret_cast<vec4 *>(out + (static_cast<int64_t>(row0 + li) * H + h) * DV + ct * 16 + 4 * lq) = w;
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int D, int DV>
+int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q, const T *kc, const T *vc,
+              const int32_t *bt, const int32_t *ts, const int32_t *tp, const int32_t *r0, const int32_t *cn,
+              const float *talk, int H, int G, int64_t qs, int window, float scale, float softcap, int mb, int64_t bs) {
+#define SWL_WM_LAUNCH(HPW)                                                                                              \
+    hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW>), grid, dim3(kWmThreads), lds, s, out, q, kc, vc, bt, ts, \
+                       tp, r0, cn, talk, H, G, qs, window, scale, softcap, mb, bs)
+    switch (hpw) {
+    case 1: SWL_WM_LAUNCH(1); break;
+    case 2: SWL_WM_LAUNCH(2); break;
+    case 4: SWL_WM_LAUNCH(4); break;
+    case 8: SWL_WM_LAUNCH(8); break;
+    default: return SWL_ERR_UNSUPPORTED;
+    }
+#undef SWL_WM_LAUNCH
+    return check_launch();
+}
+
+} // namespace swl
+
+/* 1 when swl_window_attn_tiles serves this shape (else the caller uses swl_window_attn). */
+extern "C" int swl_window_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim,
+                                               int32_t dtype) {
+    if (dtype != SWL_F16 && dtype != SWL_BF16) return 0;
+    if (num_q_heads <= 0 || num_q_heads > 32 || num_kv_heads <= 0 || num_q_heads % num_kv_heads) return 0;
+    return (dim == 64 && vdim == 64) || (dim == 128 && vdim == 128) || (dim == 128 && vdim == 64) ||
+           (dim == 64 && vdim == 128);
+}
+
+extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                     const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                                     const int32_t *tile_row0, const int32_t *tile_cnt, const float *talk,
+                                     int32_t num_tiles, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
+                                     int32_t vdim, int64_t q_tok_stride, int32_t window, float scale, float softcap,
+                                     int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
+                                     swl_stream_t stream) {
+    if (num_tiles < 0 || window < 0) return SWL_ERR_BAD_ARG;
+    if (!swl_window_attn_tiles_supported(num_q_heads, num_kv_heads, dim, vdim, dtype)) return SWL_ERR_UNSUPPORTED;
+    if (num_tiles == 0) return SWL_OK;
+    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !tile_row0 || !tile_cnt || !talk)
+        return SWL_ERR_BAD_ARG;
+    if ((q_tok_stride & 3) || (block_stride & 3) || (reinterpret_cast<uintptr_t>(q) & 7) ||
+        (reinterpret_cast<uintptr_t>(k_cache) & 7) || (reinterpret_cast<uintptr_t>(out) & 7))
+        return SWL_ERR_BAD_ARG;     // 8-byte operand loads
+    int hpw = (num_q_heads + swl::kWmWaves - 1) / swl::kWmWaves;
+    hpw = hpw <= 1 ? 1 : hpw <= 2 ? 2 : hpw <= 4 ? 4 : 8;
+    const size_t lds = static_cast<size_t>(num_q_heads) * 64 * 4 * sizeof(float);
+    const dim3 grid(static_cast<unsigned>(num_tiles));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define SWL_WM_SHAPE(DD, DDV)                                                                                             \
+    if (dim == DD && vdim == DDV)                                                                                         \
+        return swl::launch_wm<T, DD, DDV>(hpw, grid, lds, s, static_cast<T *>(out), static_cast<const T *>(q),           \
+                                          static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, \
+                                          tok_seq, tok_pos, tile_row0, tile_cnt, talk, num_q_heads, num_kv_heads,        \
+                                          q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride);
+    SWL_DISPATCH_DTYPE(dtype, T, {
+        SWL_WM_SHAPE(64, 64)
+        SWL_WM_SHAPE(128, 128)
+        SWL_WM_SHAPE(128, 64)
+        SWL_WM_SHAPE(64, 128)
+    });
+#undef SWL_WM_SHAPE
+    return SWL_ERR_UNSUPPORTED;
+}

@@ -157,8 +157,12 @@ class StepPlan:
     tok_pos: np.ndarray                 # [T] int32 position of each token in its sequence
     tok_seq: np.ndarray                 # [T] int32 block-table row of each token
     want_rows: np.ndarray               # [R] int32 rows (into the T tokens) whose logits are produced
+    # tiles of up to TILE consecutive tokens of one sequence (the matrix-core attention's unit of work)
+    tile_row0: np.ndarray = None        # [NT] int32 first token row of each tile
+    tile_cnt: np.ndarray = None         # [NT] int32 tokens in it
 
-    SEGMENTS = ("input_ids", "tok_pos", "tok_seq", "want_rows")
+    TILE = 16
+    SEGMENTS = ("input_ids", "tok_pos", "tok_seq", "want_rows", "tile_row0", "tile_cnt")
 
     def packed_layout(self):
         out, off = [], 0
@@ -205,5 +209,13 @@ def plan_step(entries: Sequence[StepEntry], vocab_size: int = None, max_position
         targets.append(int(e.start + n))
         base += n
     cat = (lambda xs: np.concatenate(xs) if xs else np.empty(0, dtype=np.int32))
-    return StepPlan(num_tokens=base, num_seqs=len(seq_ids), seq_ids_list=seq_ids, target_lens_list=targets,
+    row0, cnt, at = [], [], 0
+    for e in entries:
+        n = len(e.tokens)
+        starts = np.arange(0, n, StepPlan.TILE, dtype=np.int32)
+        row0.append(at + starts)
+        cnt.append(np.minimum(StepPlan.TILE, n - starts).astype(np.int32))
+        at += n
+    return StepPlan(tile_row0=cat(row0), tile_cnt=cat(cnt),
+                    num_tokens=base, num_seqs=len(seq_ids), seq_ids_list=seq_ids, target_lens_list=targets,
                     input_ids=cat(ids), tok_pos=cat(pos), tok_seq=cat(seq), want_rows=np.asarray(want, dtype=np.int32))

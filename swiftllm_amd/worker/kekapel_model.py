@@ -64,6 +64,11 @@ class KekapelModel:
         self._layout_pool()
         self._meta_host = self._meta_host_np = self._meta_dev = self._meta_done = None
         self.after_launch_hook = None
+        # pure-decode steps (every sequence brings one token and asks for its logits) replay a captured hipGraph, one per
+        # batch size: the step's launch geometry depends on the token count only, never on positions or block ids
+        self._decode_graphs = {}
+        self._graph_pool = None
+        self.graph_captures = 0
         # tests set these to lists: the fp32 stream after every layer run / the logits of every step
         self.layer_tap = None
         self.logits_tap = None
@@ -153,6 +158,8 @@ class KekapelModel:
             self.kv_swap = torch.zeros((ecfg.num_cpu_blocks, self.block_elems), dtype=self.dtype, pin_memory=pin)
         except RuntimeError:
             self.kv_swap = torch.zeros((ecfg.num_cpu_blocks, self.block_elems), dtype=self.dtype)
+        self._decode_graphs.clear()     # (captured against the previous pool and block table)
+        self._graph_pool = None
         self.gpu_block_manager = BlockManager("GPU", num_blocks, ecfg.max_seqs_in_block_table, ecfg.max_blocks_per_seq,
                                               ecfg.block_size, self.device)
         self.cpu_block_manager = BlockManager("CPU", ecfg.num_cpu_blocks, ecfg.max_seqs_in_block_table,
@@ -198,7 +205,7 @@ class KekapelModel:
         for i, s in enumerate(subs):
             if s.kind == "mixer":
                 y = s.op.forward(h, pool, self.pool_slices[s.run] if use_pool else None, block_table, dev["tok_seq"],
-                                 dev["tok_pos"])
+                                 dev["tok_pos"], (dev["tile_row0"], dev["tile_cnt"]))
             else:
                 y = s.op.forward(h)
             nxt = subs[i + 1] if i + 1 < len(subs) else None
@@ -230,13 +237,47 @@ class KekapelModel:
         if not ignore_kvcache:
             self.gpu_block_manager.allocate_blocks_for_seqs(plan.seq_ids_list, plan.target_lens_list)
         dev = self._upload_plan(plan)
-        x = self._run_stack(dev, not ignore_kvcache)
-        if plan.want_rows.size == 0:
-            return torch.empty((0, cfg.vocab_size), dtype=self.dtype, device=self.device)
-        logits = self._logits(x, dev["want_rows"])
+        if (getattr(self.engine_config, "use_hip_graph", False) and not ignore_kvcache and self.layer_tap is None
+                and plan.num_tokens == plan.num_seqs == plan.want_rows.size):
+            logits = self._step_decode_graph(plan, dev)
+        else:
+            x = self._run_stack(dev, not ignore_kvcache)
+            if plan.want_rows.size == 0:
+                return torch.empty((0, cfg.vocab_size), dtype=self.dtype, device=self.device)
+            logits = self._logits(x, dev["want_rows"])
         if self.logits_tap is not None:
-            self.logits_tap.append(logits)
+            self.logits_tap.append(logits.clone())
         return logits
+
+    _MAX_DECODE_GRAPHS = 64
+
+    def _step_decode_graph(self, plan: StepPlan, dev: dict) -> torch.Tensor:
+        """Replay (capturing it first, once per batch size) the whole pure-decode step. The metadata buffer has a fixed
+        address and a layout that depends on the token count only, so a replay reads this step's tokens, positions and
+        block-table rows from where the capture did. The returned logits are the graph's own output buffer: valid until
+        the next replay of the same graph."""
+        key = plan.num_tokens
+        entry = self._decode_graphs.pop(key, None)
+        if entry is not None and entry[2] != self._meta_dev.data_ptr():
+            entry = None        # the metadata buffer was re-allocated: the capture points at the old one
+        if entry is None:
+            self.graph_captures += 1
+            warm = torch.cuda.Stream()      # one eager run first: nothing may be lazily initialised under capture
+            warm.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(warm):
+                self._logits(self._run_stack(dev, True), dev["want_rows"])
+            torch.cuda.current_stream().wait_stream(warm)
+            while len(self._decode_graphs) >= self._MAX_DECODE_GRAPHS:
+                self._decode_graphs.pop(next(iter(self._decode_graphs)))
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                out = self._logits(self._run_stack(dev, True), dev["want_rows"])
+            entry = (graph, out, self._meta_dev.data_ptr())
+        self._decode_graphs[key] = entry
+        entry[0].replay()
+        return entry[1]
 
     @torch.inference_mode()
     def forward(self, input_ids_list: List[List[int]], seq_ids_list: List[int], decoding_seq_lens_list: List[int],

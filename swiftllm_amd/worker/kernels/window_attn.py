@@ -39,16 +39,38 @@ def qknorm_and_store_kv(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: torch.T
               _hip.dtype_code3(qkv.dtype), _hip.stream())
 
 
+# Steps with at least this many tokens go to the matrix-core kernel (tiles of 16 queries); smaller ones — decode batches — to
+# the per-token kernel, whose workgroups are not mostly padding there.
+TILES_MIN_TOKENS = 48
+
+
+def tiles_supported(mixer, dtype: torch.dtype) -> bool:
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
+    return bool(_hip.load().swl_window_attn_tiles_supported(mixer.num_q_heads, mixer.num_kv_heads, mixer.head_dim,
+                                                            mixer.value_dim, _hip.dtype_code(dtype)))
+
+
 def window_attention(qkv: torch.Tensor, talk: torch.Tensor, pool: torch.Tensor, pool_slice: PoolSlice,
-                     block_table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, mixer) -> torch.Tensor:
+                     block_table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, mixer,
+                     tiles=None) -> torch.Tensor:
     """-> [T, heads * vdim]. The queries are the (already normalised) first columns of qkv; keys and values come from the
-    pool, which already holds this step's tokens."""
+    pool, which already holds this step's tokens. `tiles` = (tile_row0, tile_cnt) device arrays: the step cut into runs of
+    up to 16 consecutive tokens of one sequence — given, and the shape served, the matrix-core kernel runs."""
     _hip.require_gpu_tensor(qkv, "qkv")
     assert talk.dtype == torch.float32 and talk.is_contiguous() and talk.shape == (mixer.num_q_heads, mixer.num_q_heads)
     assert pool.is_contiguous() and pool.dtype == qkv.dtype
     n = qkv.shape[0]
     out = torch.empty((n, mixer.num_q_heads * mixer.value_dim), dtype=qkv.dtype, device=qkv.device)
     esize = pool.element_size()
+    if tiles is not None and n >= TILES_MIN_TOKENS and tiles_supported(mixer, qkv.dtype):
+        row0, cnt = tiles
+        _hip.call("swl_window_attn_tiles", _hip.ptr(out), _hip.ptr(qkv), pool.data_ptr() + pool_slice.k_offset * esize,
+                  pool.data_ptr() + pool_slice.v_offset * esize, _hip.ptr(block_table), _hip.ptr(tok_seq),
+                  _hip.ptr(tok_pos), _hip.ptr(row0), _hip.ptr(cnt), _hip.ptr(talk), row0.shape[0], mixer.num_q_heads,
+                  mixer.num_kv_heads, mixer.head_dim, mixer.value_dim, qkv.stride(0), mixer.window, float(mixer.scale),
+                  float(mixer.softcap), block_table.shape[1], pool.shape[1], _hip.dtype_code(qkv.dtype), _hip.stream())
+        return out
     _hip.call("swl_window_attn", _hip.ptr(out), _hip.ptr(qkv), pool.data_ptr() + pool_slice.k_offset * esize,
               pool.data_ptr() + pool_slice.v_offset * esize, _hip.ptr(block_table), _hip.ptr(tok_seq), _hip.ptr(tok_pos),
               _hip.ptr(talk), n, mixer.num_q_heads, mixer.num_kv_heads, mixer.head_dim, mixer.value_dim, qkv.stride(0),

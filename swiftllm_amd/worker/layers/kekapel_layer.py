@@ -23,14 +23,14 @@ class KekapelAttention:
     def __init__(self, layer_config, weight, eps: float, skinny: bool):
         self.mixer, self.w, self.eps, self.skinny = layer_config.mixer, weight, eps, skinny
 
-    def forward(self, h: torch.Tensor, pool, pool_slice, block_table, tok_seq, tok_pos) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, pool, pool_slice, block_table, tok_seq, tok_pos, tiles=None) -> torch.Tensor:
         qkv = _project(h, self.w.qkv, self.skinny)
         qknorm_and_store_kv(qkv, self.w.q_norm, self.w.k_norm, pool, pool_slice, block_table, tok_seq, tok_pos,
                             self.mixer, self.eps)
         if pool is None:    # memory profiling: the attention's output buffer without its reads
             attn = torch.zeros((h.shape[0], self.mixer.num_q_heads * self.mixer.value_dim), dtype=h.dtype, device=h.device)
         else:
-            attn = window_attention(qkv, self.w.talk, pool, pool_slice, block_table, tok_seq, tok_pos, self.mixer)
+            attn = window_attention(qkv, self.w.talk, pool, pool_slice, block_table, tok_seq, tok_pos, self.mixer, tiles)
         return _project(attn, self.w.o, self.skinny)
 
 

@@ -124,10 +124,12 @@ def test_moe_router_and_experts(experts, top):
     assert (got.cpu().double() - want).abs().max() < 2e-5
 
 
-def _attention_case(heads, kv_heads, dim, vdim, window, n, softcap, seed, standout=None, dtype=torch.float32):
+def _attention_case(heads, kv_heads, dim, vdim, window, n, softcap, seed, standout=None, dtype=torch.float32, tiled=False,
+                    cuts=None):
     """One mixer over a sequence of n tokens held in scattered blocks, fed as two portions and one decoded token, against
     the dense-mask oracle. standout = (query, key): that pair's score is made to dominate its row."""
     from swiftllm_amd.model_config import KekapelMixerConfig
+    from swiftllm_amd.worker.kernels import window_attn
     from swiftllm_amd.worker.kernels.window_attn import PoolSlice, qknorm_and_store_kv, window_attention
     g = torch.Generator().manual_seed(seed)
     mxd = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": 0.35, "softcap": softcap,
@@ -163,13 +165,24 @@ def _attention_case(heads, kv_heads, dim, vdim, window, n, softcap, seed, stando
     pos = torch.arange(n, dtype=torch.int32).cuda()
     table = table.cuda()
     out = []
-    cuts = [0, max(1, n // 3), n - 1, n] if n > 2 else [0, n]
-    for a, b in zip(cuts[:-1], cuts[1:]):
-        if a == b:
-            continue
-        part = qkv[a:b].contiguous()
-        qknorm_and_store_kv(part, qn.cuda(), kn.cuda(), pool, sl, table, seq[a:b], pos[a:b], mixer, eps)
-        out.append(window_attention(part, talk.cuda(), pool, sl, table, seq[a:b], pos[a:b], mixer))
+    if cuts is None:
+        cuts = [0, max(1, n // 3), n - 1, n] if n > 2 else [0, n]
+    saved = window_attn.TILES_MIN_TOKENS
+    window_attn.TILES_MIN_TOKENS = 1 if tiled else saved
+    try:
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            if a == b:
+                continue
+            part = qkv[a:b].contiguous()
+            qknorm_and_store_kv(part, qn.cuda(), kn.cuda(), pool, sl, table, seq[a:b], pos[a:b], mixer, eps)
+            tiles = None
+            if tiled:
+                assert window_attn.tiles_supported(mixer, dtype)
+                starts = torch.arange(0, b - a, 16, dtype=torch.int32)
+                tiles = (starts.cuda(), torch.clamp(b - a - starts, max=16).to(torch.int32).cuda())
+            out.append(window_attention(part, talk.cuda(), pool, sl, table, seq[a:b], pos[a:b], mixer, tiles))
+    finally:
+        window_attn.TILES_MIN_TOKENS = saved
     got = torch.cat(out).cpu().double()
     return got, want
 
@@ -182,6 +195,35 @@ def test_window_attention_against_dense_mask(heads, kv_heads, dim, vdim, window,
     assert (got - want).abs().max() < 2e-5
     got, want = _attention_case(heads, kv_heads, dim, vdim, window, n, None, seed=n + 1, dtype=torch.bfloat16)
     assert (got - want).abs().max() < 8e-2     # (q and k are rounded to bfloat16 after their norms; scores reach +-20 here)
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,window,n", [
+    (6, 3, 64, 64, 40, 150), (8, 2, 128, 128, 9, 70), (16, 4, 128, 64, 64, 131), (32, 8, 64, 64, 33, 90),
+    (5, 5, 64, 128, 200, 100), (1, 1, 64, 64, 16, 49), (3, 1, 128, 128, 1, 40), (32, 4, 128, 128, 17, 50)])
+@pytest.mark.parametrize("dtype,atol", [(torch.float16, 4e-3), (torch.bfloat16, 3.2e-2)])
+def test_tiled_attention_matches_the_per_token_kernel(heads, kv_heads, dim, vdim, window, n, dtype, atol):
+    """The matrix-core kernel (tiles of 16 queries, portions cut at odd places, a decoded token as a tile of one) against
+    the per-token kernel on the same 16-bit inputs: they differ by rounding only."""
+    cuts = [0, 5, 5 + 37, n - 1, n] if n > 45 else [0, 3, n - 1, n]
+    for cap in (7.0, None):
+        kw = dict(softcap=cap, seed=n + heads, dtype=dtype, cuts=cuts)
+        tiled, want = _attention_case(heads, kv_heads, dim, vdim, window, n, tiled=True, **kw)
+        plain, _ = _attention_case(heads, kv_heads, dim, vdim, window, n, tiled=False, **kw)
+        assert (tiled - plain).abs().max() < atol * max(1.0, float(plain.abs().max()))
+        assert (tiled - want).abs().max() < 0.3     # (16-bit q and k after their norms: uncapped scores reach +-45)
+
+
+@pytest.mark.parametrize("window,n", [(9, 60), (16, 70), (40, 150), (64, 131)])
+def test_tiled_window_edges_show_in_the_output(window, n):
+    for qi in (n - 1, n - 2, 48 if n > 48 + 1 else n - 3, 17):
+        for back in (window - 1, window):
+            kj = qi - back
+            if kj < 0:
+                continue
+            args = (4, 2, 64, 64, window, n, 30.0)
+            kw = dict(seed=qi * 7 + back, standout=(qi, kj), dtype=torch.float16, cuts=[0, n - 1, n])
+            got, want = _attention_case(*args, tiled=True, **kw)
+            assert (got - want).abs().max() < 2e-2, (qi, kj)
 
 
 @pytest.mark.parametrize("window,n", [(9, 60), (16, 70), (40, 150), (64, 131)])
@@ -244,6 +286,34 @@ def test_decoding_and_portions_match_the_whole_prompt(tmp_path, default_case, dt
         assert at == len(toks)
         assert rel_err(torch.cat(rows), want) < tol, sizes
         model.free_seqs_resources([3])
+
+
+def test_decode_graph_replays_match_eager_steps(tmp_path, default_case):
+    """Pure-decode steps replay a captured hipGraph: several replays, with eager prompt portions and a changing batch in
+    between, every one against the oracle."""
+    cfg, W, toks, want, _ = default_case
+    from swiftllm_amd import EngineConfig, build_model
+    path = write_model(tmp_path / "g", cfg, W)
+    ecfg = EngineConfig(model_path=path, use_dummy=False, block_size=16, gpu_mem_utilization=0.9, num_cpu_blocks=0,
+                        max_seqs_in_block_table=4, max_blocks_per_seq=16, max_batch_size=4, max_tokens_in_batch=256,
+                        dtype="float32", use_hip_graph=True)
+    model = build_model(ecfg)
+    model.load_weights()
+    model.init_kvcache_and_swap(24)
+    other = tokens_for(cfg, 60, 31)
+    want2 = O.forward(cfg, W, other)
+    model.step([entry(0, toks[:20], 0, want=[])])
+    got0, got1 = [], []
+    for i in range(20, 30):         # batch 1: one capture, ten replays
+        got0.append(model.step([entry(0, toks[i:i + 1], i)]).clone())
+    model.step([entry(1, other[:33], 0, want=[])])      # an eager portion in between
+    for i in range(12):             # batch 2: another capture
+        out = model.step([entry(0, toks[30 + i:31 + i], 30 + i), entry(1, other[33 + i:34 + i], 33 + i)])
+        got0.append(out[:1].clone())
+        got1.append(out[1:].clone())
+    assert model.graph_captures == 2
+    assert rel_err(torch.cat(got0), want[20:42]) < F32_TOL
+    assert rel_err(torch.cat(got1), want2[33:45]) < F32_TOL
 
 
 def test_unequal_batches_and_reused_blocks_and_rows(tmp_path, default_case):
