@@ -509,7 +509,7 @@ int swl_add_layernorm(float *x, const void *y, float mult, const float *w1, cons
 /* ---- per-head q/k RMS norm + paged KV store ---------------------------------------------------------------------------
  * qkv[T, tok_stride] = [q heads | k heads | v heads] of one fused projection. q heads are normalised in place (weight q_w
  * [dim], shared by the heads); k heads are normalised (k_w) into the K pool (block b = [kv_heads, 16, dim] at k_cache + b * block_stride
- * elements); v heads are copied into the V pool (block b = [kv_heads, 16, vdim] at v_cache + b * block_stride), block
+ * elements); v heads are copied into the V pool (block b = [kv_heads, vdim, 16], TRANSPOSED, at v_cache + b * block_stride), block
  * block_table[tok_seq[t]][tok_pos[t] / 16], slot tok_pos[t] % 16.
  * k_cache == NULL: only the query norm (memory-profiling runs). dtype may be SWL_F32. */
 int swl_qknorm_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_cache, void *v_cache,
@@ -530,14 +530,16 @@ int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v
 /* The matrix-core form for 16-bit dtypes and head sizes 64 / 128: the step's tokens come as tiles of up to 16 consecutive
  * tokens of one sequence (tile_row0[i] = first token row, tile_cnt[i] = tokens; a decoded token is a tile of one). Same
  * arithmetic as swl_window_attn up to rounding (fp32 scores and weights; weights enter the value product as hi + lo 16-bit
- * terms). swl_window_attn_tiles_supported: 1 when it serves the shape. */
+ * terms). key_splits > 1 (few tiles, long windows: decode batches): each tile's pages are shared out over that many
+ * workgroups, whose partial results (scratch: key_splits * num_tokens * H * (vdim + 2) floats, 16-byte aligned) a second launch
+ * combines. swl_window_attn_tiles_supported: 1 when it serves the shape. */
 int swl_window_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int32_t dtype);
 int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
                           const int32_t *tok_seq, const int32_t *tok_pos, const int32_t *tile_row0,
                           const int32_t *tile_cnt, const float *talk, int32_t num_tiles, int32_t num_q_heads,
                           int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window,
-                          float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
-                          swl_stream_t stream);
+                          float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride,
+                          int32_t key_splits, float *scratch, int64_t num_tokens, int32_t dtype, swl_stream_t stream);
 
 /* ---- PolyNorm activation: out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row ---------- */
 int swl_polynorm(void *out, const void *z, float a, float b, float c, float e, float eps, int64_t num_rows, int32_t ff,
@@ -552,6 +554,13 @@ int swl_moe_route(int32_t *idx_out, float *w_out, const void *h, const float *ro
                   int64_t num_tokens, int32_t width, int32_t experts, int32_t top, int32_t dtype, swl_stream_t stream);
 int swl_moe_gate_up(void *y, const void *h, const void *gate_up, const int32_t *expert_idx, int64_t num_tokens,
                     int32_t width, int32_t ff, int32_t top, float limit, int32_t dtype, swl_stream_t stream);
+/* Large steps (prompt portions): assignments are sorted by expert and every expert's rows go through the library GEMM;
+ * swl_glu_clamp: y[r][f] = act of [gate | up] product rows gate_up[r][2 ff]; swl_moe_combine: out[t] = sum_j w[t][j] *
+ * rows[where[t * top + j]] (fp32, fixed order). dtype may be SWL_F32. */
+int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t dtype,
+                  swl_stream_t stream);
+int swl_moe_combine(void *out, const void *rows, const int64_t *where, const float *expert_w, int64_t num_tokens,
+                    int32_t width, int32_t top, int32_t dtype, swl_stream_t stream);
 int swl_moe_down_combine(void *out, const void *y, const void *down, const int32_t *expert_idx, const float *expert_w,
                          int64_t num_tokens, int32_t width, int32_t ff, int32_t top, int32_t dtype, swl_stream_t stream);
 

@@ -101,10 +101,12 @@ SIGNATURES = {
     "swl_window_attn": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32, _I32,
                         _I64, _I32, _P],
     "swl_window_attn_tiles": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32,
-                              _I32, _I64, _I32, _P],
+                              _I32, _I64, _I32, _P, _I64, _I32, _P],
     "swl_polynorm": [_P, _P, _F32, _F32, _F32, _F32, _F32, _I64, _I32, _I32, _P],
     "swl_moe_route": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
     "swl_moe_gate_up": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _P],
+    "swl_glu_clamp": [_P, _P, _I64, _I32, _F32, _I32, _P],
+    "swl_moe_combine": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _P],
     "swl_moe_down_combine": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
 }
 # Entry points that do not follow the "int rc = f(...)" convention.

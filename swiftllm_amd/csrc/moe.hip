@@ -13,8 +13,46 @@
 
 namespace swl {
 
+__device__ __forceinline__ bool aligned16_dev(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 constexpr int kMoeThreads = 256;
 constexpr int kMoeWaves = kMoeThreads / 64;
+
+// Per-lane share of sum_i x[i] * w[i] over a row of n elements (x fp32 in LDS, w in global memory); the caller reduces
+// over the wave. 16-bit rows whose length is a multiple of 8 are read 16 bytes per lane.
+template <typename T>
+__device__ __forceinline__ float lane_dot(const float *x, const T *w, int n, int lane) {
+    float a = 0.f;
+    if constexpr (sizeof(T) == 2) {
+        if ((n & 7) == 0 && aligned16_dev(w)) {
+            for (int i = lane * 8; i < n; i += 64 * 8) {
+                const vec8_t<T> v = load8(w + i);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a += x[i + j] * to_f(v[j]);
+            }
+            return a;
+        }
+    }
+    for (int i = lane; i < n; i += 64) a += x[i] * to_f(w[i]);
+    return a;
+}
+// The same with both rows in global memory.
+template <typename T>
+__device__ __forceinline__ float lane_dot2(const T *x, const T *w, int n, int lane) {
+    float a = 0.f;
+    if constexpr (sizeof(T) == 2) {
+        if ((n & 7) == 0 && aligned16_dev(w) && aligned16_dev(x)) {
+            for (int i = lane * 8; i < n; i += 64 * 8) {
+                const vec8_t<T> v = load8(w + i), u = load8(x + i);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a += to_f(u[j]) * to_f(v[j]);
+            }
+            return a;
+        }
+    }
+    for (int i = lane; i < n; i += 64) a += to_f(x[i]) * to_f(w[i]);
+    return a;
+}
 
 template <typename T>
 __global__ __launch_bounds__(kMoeThreads) void moe_route_kernel(int32_t *idx_out, float *w_out, const T *h,
@@ -90,12 +128,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_gate_up_kernel(T *y, const T 
     const int f0 = blockIdx.y * 64;
     for (int f = f0 + wave; f < min(ff, f0 + 64); f += kMoeWaves) {
         const T *rg = wg + static_cast<int64_t>(f) * width, *ru = wu + static_cast<int64_t>(f) * width;
-        float g = 0.f, u = 0.f;
-        for (int i = lane; i < width; i += 64) {
-            const float x = hf[i];
-            g += x * to_f(rg[i]);
-            u += x * to_f(ru[i]);
-        }
+        float g = lane_dot(hf, rg, width, lane), u = lane_dot(hf, ru, width, lane);
         g = wave_allreduce_sum(g);
         u = wave_allreduce_sum(u);
         if (lane == 0) {
@@ -121,16 +154,69 @@ __global__ __launch_bounds__(kMoeThreads) void moe_down_combine_kernel(T *out, c
             const int e = expert_idx[t * top + j];
             const T *wr = down + (static_cast<int64_t>(e) * width + c) * ff;
             const T *yr = y + (t * top + j) * ff;
-            float a = 0.f;
-            for (int i = lane; i < ff; i += 64) a += to_f(yr[i]) * to_f(wr[i]);
-            a = wave_allreduce_sum(a);
+            float a = wave_allreduce_sum(lane_dot2(yr, wr, ff, lane));
             total += expert_w[t * top + j] * a;
         }
         if (lane == 0) out[t * width + c] = to_t<T>(total);
     }
 }
 
+// y[r][f] = act(gu[r][f], gu[r][ff + f]) for rows of [gate | up] products that came from a library GEMM
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void glu_clamp_kernel(T *y, const T *gu, int64_t total, int ff, float limit) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kMoeThreads + threadIdx.x;
+    if (i >= total) return;
+    const int64_t r = i / ff;
+    const int f = static_cast<int>(i - r * ff);
+    float g = fminf(to_f(gu[r * 2 * ff + f]), limit);
+    const float u = fminf(fmaxf(to_f(gu[r * 2 * ff + ff + f]), -limit), limit);
+    const float sg = 1.0f / (1.0f + expf(-1.702f * g));
+    y[i] = to_t<T>(g * sg * (u + 1.0f));
+}
+
+// out[t] = sum_j w[t][j] * rows[where[t * top + j]]  (fp32 sum in the order j = 0, 1, ...)
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void moe_combine_kernel(T *out, const T *rows, const int64_t *where,
+                                                                  const float *w, int width, int top) {
+    const int64_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += kMoeThreads) {
+        float a = 0.f;
+        for (int j = 0; j < top; ++j) a += w[t * top + j] * to_f(rows[where[t * top + j] * width + c]);
+        out[t * width + c] = to_t<T>(a);
+    }
+}
+
 } // namespace swl
+
+extern "C" int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t dtype,
+                             swl_stream_t stream) {
+    if (num_rows < 0 || ff <= 0) return SWL_ERR_BAD_ARG;
+    if (num_rows == 0) return SWL_OK;
+    if (!y || !gate_up) return SWL_ERR_BAD_ARG;
+    const int64_t total = num_rows * ff;
+    const int64_t blocks = (total + swl::kMoeThreads - 1) / swl::kMoeThreads;
+    if (blocks > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::glu_clamp_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(swl::kMoeThreads), 0,
+                           static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(gate_up), total,
+                           ff, limit);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_moe_combine(void *out, const void *rows, const int64_t *where, const float *expert_w,
+                               int64_t num_tokens, int32_t width, int32_t top, int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || top <= 0) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!out || !rows || !where || !expert_w) return SWL_ERR_BAD_ARG;
+    if (num_tokens > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::moe_combine_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kMoeThreads), 0,
+                           static_cast<hipStream_t>(stream), static_cast<T *>(out), static_cast<const T *>(rows), where,
+                           expert_w, width, top);
+    });
+    return swl::check_launch();
+}
 
 extern "C" int swl_moe_route(int32_t *idx_out, float *w_out, const void *h, const float *router, const float *bias,
                              int64_t num_tokens, int32_t width, int32_t experts, int32_t top, int32_t dtype,

@@ -6,7 +6,8 @@
 // norm weight is shared by all heads (plain weight, not one-plus).
 //
 // Pool layout: block b of a layer run's keys starts at k_cache + b * block_stride and holds [kv_heads, 16, dim]; its values
-// start at v_cache + b * block_stride and hold [kv_heads, 16, vdim] (block_stride in elements: a block of the pool may hold the
+// start at v_cache + b * block_stride and hold [kv_heads, vdim, 16] — TRANSPOSED, the 16 tokens of a column contiguous, which is
+// how the matrix-core attention wants its value operand (block_stride in elements: a block of the pool may hold the
 // keys and values of several layer runs side by side, so that swapping moves one contiguous piece per block).
 #include "swl_common.h"
 
@@ -51,7 +52,7 @@ __global__ __launch_bounds__(kQkThreads) void qknorm_store_kv_kernel(
         const T *vsrc = row + static_cast<int64_t>(H + G) * d;
         for (int i = threadIdx.x; i < G * dv; i += kQkThreads) {
             const int g = i / dv, c = i - g * dv;
-            v_cache[blk * block_stride + (static_cast<int64_t>(g) * kQkBlock + off) * dv + c] = vsrc[i];
+            v_cache[blk * block_stride + (static_cast<int64_t>(g) * dv + c) * kQkBlock + off] = vsrc[i];    // transposed page
         }
     }
 }

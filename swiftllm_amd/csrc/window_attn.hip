@@ -126,8 +126,9 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
                 float a = acc[i] * alpha[h];
                 const float *ph = p + h * kWaChunk;
                 for (int j = 0; j < cn; ++j) {
-                    const T *vr = v_cache + kbase[j] * block_stride + (static_cast<int64_t>(g) * kWaBlock + koff[j]) * dv;
-                    a += ph[j] * to_f(vr[col]);
+                    // (a page keeps its values transposed: [kv head][column][16 tokens])
+                    const T *vr = v_cache + kbase[j] * block_stride + (static_cast<int64_t>(g) * dv + col) * kWaBlock;
+                    a += ph[j] * to_f(vr[koff[j]]);
                 }
                 acc[i] = a;
             }

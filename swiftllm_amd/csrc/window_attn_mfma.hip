@@ -56,10 +56,11 @@ __device__ __forceinline__ float fast_tanh(float x) {
 }
 
 template <typename T, int D, int DV, int HPW>
-__global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
+__global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk, int H, int G,
-    int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride) {
+    int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
+    float *part_o, float *part_ml, int64_t num_tokens) {
     extern __shared__ float s_lds[];    // [H][64 lanes][4]
     constexpr int CT = DV / 16;         // 16-column tiles of the value head
     constexpr float kLog2e = 1.4426950408889634f;
@@ -74,7 +75,12 @@ __global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
     const int qpos = p0 + li;                        // this lane's query position (meaningful when li < cnt)
     const bool qok = li < cnt;
     const int lo_first = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
-    const int kb0 = lo_first / kWmTile, kb1 = (p0 + cnt - 1) / kWmTile;
+    int kb0 = lo_first / kWmTile, kb1 = (p0 + cnt - 1) / kWmTile;
+    if (gridDim.y > 1) {    // key split: this workgroup takes a contiguous share of the tile's pages (possibly none)
+        const int per = (kb1 - kb0 + static_cast<int>(gridDim.y)) / static_cast<int>(gridDim.y);
+        kb0 += per * static_cast<int>(blockIdx.y);
+        kb1 = min(kb1, kb0 + per - 1);
+    }
     const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
 
     float4_t acc[HPW][CT];
@@ -88,25 +94,67 @@ __global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
     }
     // the query row this lane feeds as B operand of S^T = K Q^T: row li of the tile (rows past cnt: the tile's last row)
     const T *qrow = q + static_cast<int64_t>(row0 + (qok ? li : cnt - 1)) * q_tok_stride;
+    // Registers allowing (PIPE), the query fragments stay resident and the next page's key fragments are fetched while this
+    // page's mix / softmax / value products run; the value fragments of a page are requested before its score products.
+    constexpr int KS = D / 16;
+    constexpr bool PIPE = HPW * D <= 512 && HPW * DV <= 512;
+    T qf[PIPE ? HPW : 1][KS][4], kf[PIPE ? HPW : 1][KS][4];
+    auto fetch_k = [&](int kb) {
+        const T *kblk = k_cache + static_cast<int64_t>(bt[kb]) * block_stride;
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+            const int g = min(h0 + hh, H - 1);
+            const T *kr = kblk + (static_cast<int64_t>(g / rep) * kWmTile + li) * D + 4 * lq;    // A: key li, dims 4 lq ..
+#pragma unroll
+            for (int e = 0; e < KS; ++e) load4(kf[PIPE ? hh : 0][e], kr + e * 16);
+        }
+    };
+    if constexpr (PIPE) {
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+            const int g = min(h0 + hh, H - 1);
+#pragma unroll
+            for (int e = 0; e < KS; ++e) load4(qf[hh][e], qrow + g * D + 4 * lq + e * 16);     // B: query li
+        }
+        if (kb0 <= kb1) fetch_k(kb0);
+    }
 
     for (int kb = kb0; kb <= kb1; ++kb) {
         const int64_t blk = bt[kb];
         const T *kblk = k_cache + blk * block_stride;
         const T *vblk = v_cache + blk * block_stride;
+        // value fragments of this page, A operand of O^T += V^T P^T: V^T[col ct * 16 + li][keys 4 lq .. 4 lq + 3] — the pool keeps
+        // a page's values transposed ([kv head][column][16 keys]), so this is one 8-byte load
+        T vfrag[PIPE ? HPW : 1][CT][4];
+        auto fetch_v = [&](int hh) {
+            const int kv = min(h0 + hh, H - 1) / rep;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+                load4(vfrag[PIPE ? hh : 0][ct], vblk + (static_cast<int64_t>(kv) * DV + ct * 16 + li) * kWmTile + 4 * lq);
+        };
+        if constexpr (PIPE) {
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) fetch_v(hh);
+        }
         // ---- 1. capped scores of this wave's heads -> LDS -------------------------------------------------------------------
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int g = h0 + hh;
             if (g < H) {
-                const T *kr = kblk + (static_cast<int64_t>(g / rep) * kWmTile + li) * D + 4 * lq;   // A: key li, dims 4 lq ..
-                const T *qr = qrow + g * D + 4 * lq;                                                   // B: query li
                 float4_t st = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (PIPE) {
 #pragma unroll
-                for (int e = 0; e < D; e += 16) {
-                    T a[4], b[4];
-                    load4(a, kr + e);
-                    load4(b, qr + e);
-                    st = mfma16(a, b, st);
+                    for (int e = 0; e < KS; ++e) st = mfma16(kf[hh][e], qf[hh][e], st);
+                } else {
+                    const T *kr = kblk + (static_cast<int64_t>(g / rep) * kWmTile + li) * D + 4 * lq;
+                    const T *qr = qrow + g * D + 4 * lq;
+#pragma unroll
+                    for (int e = 0; e < KS; ++e) {
+                        T a[4], b[4];
+                        load4(a, kr + e * 16);
+                        load4(b, qr + e * 16);
+                        st = mfma16(a, b, st);
+                    }
                 }
                 mfma_results_ready<4>(st);
                 // st[r] = S^T[key 4 lq + r][query li]
@@ -120,6 +168,9 @@ __global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
             }
         }
         __syncthreads();
+        if constexpr (PIPE) {
+            if (kb < kb1) fetch_k(kb + 1);
+        }
         // ---- 2. mix, mask, online softmax; 3. O^T += V^T P^T for this wave's heads ------------------------------------------
         const int kpos0 = kb * kWmTile + 4 * lq;     // position of this lane's key r = 0
         bool ok[4];
@@ -143,8 +194,6 @@ __global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
                 for (int r = 0; r < 4; ++r) mixed[hh][r] += tw * sv[r];
             }
         }
-        int prev_kv = -1;
-        T vfrag[CT][4];
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int h = h0 + hh;
@@ -167,22 +216,17 @@ __global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
                     plo[r] = to_t<T>(pv - to_f(phi[r]));
                 }
                 lrun[hh] = lrun[hh] * alpha + psum;
-                const int kv = h / rep;
-                if (kv != prev_kv) {    // (wave-uniform) A operand: V^T[col ct * 16 + li][key 4 lq + r]
-                    prev_kv = kv;
-#pragma unroll
-                    for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            vfrag[ct][r] = vblk[(static_cast<int64_t>(kv) * kWmTile + 4 * lq + r) * DV + ct * 16 + li];
-                }
+                const bool rescale = !__all(alpha == 1.0f);     // (wave-uniform) most pages after the first leave the maxima alone
+                if constexpr (!PIPE) fetch_v(hh);
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     float4_t o = acc[hh][ct];
+                    if (rescale) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o[r] *= alpha;
-                    o = mfma16(vfrag[ct], phi, o);
-                    o = mfma16(vfrag[ct], plo, o);
+                        for (int r = 0; r < 4; ++r) o[r] *= alpha;
+                    }
+                    o = mfma16(vfrag[PIPE ? hh : 0][ct], phi, o);
+                    o = mfma16(vfrag[PIPE ? hh : 0][ct], plo, o);
                     acc[hh][ct] = o;
                 }
             }
@@ -197,6 +241,20 @@ __global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
             float l = lrun[hh];
             l += __shfl_xor(l, 16, 64);
             l += __shfl_xor(l, 32, 64);
+            if (gridDim.y > 1) {    // partial result of this key share: unnormalised O, running maximum, sum
+                const int64_t slot = (static_cast<int64_t>(blockIdx.y) * num_tokens + row0 + li) * H + h;
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    float4_t o = acc[hh][ct];
+                    mfma_results_ready<4>(o);
+                    if (qok) *reinterpret_cast<float4_t *>(part_o + slot * DV + ct * 16 + 4 * lq) = o;
+                }
+                if (qok && lq == 0) {
+                    part_ml[slot * 2] = mrun[hh];
+                    part_ml[slot * 2 + 1] = l;
+                }
+                continue;
+            }
             const float inv = 1.0f / l;
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
@@ -214,13 +272,32 @@ __global__ __launch_bounds__(kWmThreads) void window_attn_mfma_kernel(
     }
 }
 
+// out[t][h][:] = sum_s e^{m_s - M} O_s / sum_s e^{m_s - M} l_s over the key shares s (a share without keys has l = 0)
+template <typename T>
+__global__ __launch_bounds__(256) void window_attn_combine_kernel(T *out, const float *part_o, const float *part_ml,
+                                                                  int64_t rows, int dv, int nsplit) {
+    const int64_t row = blockIdx.x;     // (token, head)
+    float mx = kNegBig;
+    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_ml[(s * rows + row) * 2]);
+    float den = 0.f;
+    for (int s = 0; s < nsplit; ++s)
+        den += expf(part_ml[(s * rows + row) * 2] - mx) * part_ml[(s * rows + row) * 2 + 1];
+    for (int c = threadIdx.x; c < dv; c += blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < nsplit; ++s)
+            a += expf(part_ml[(s * rows + row) * 2] - mx) * part_o[(s * rows + row) * dv + c];
+        out[row * dv + c] = to_t<T>(a / den);
+    }
+}
+
 template <typename T, int D, int DV>
 int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q, const T *kc, const T *vc,
               const int32_t *bt, const int32_t *ts, const int32_t *tp, const int32_t *r0, const int32_t *cn,
-              const float *talk, int H, int G, int64_t qs, int window, float scale, float softcap, int mb, int64_t bs) {
+              const float *talk, int H, int G, int64_t qs, int window, float scale, float softcap, int mb, int64_t bs,
+              float *po, float *pml, int64_t nt) {
 #define SWL_WM_LAUNCH(HPW)                                                                                              \
     hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW>), grid, dim3(kWmThreads), lds, s, out, q, kc, vc, bt, ts, \
-                       tp, r0, cn, talk, H, G, qs, window, scale, softcap, mb, bs)
+                       tp, r0, cn, talk, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt)
     switch (hpw) {
     case 1: SWL_WM_LAUNCH(1); break;
     case 2: SWL_WM_LAUNCH(2); break;
@@ -229,6 +306,11 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
     default: return SWL_ERR_UNSUPPORTED;
     }
 #undef SWL_WM_LAUNCH
+    if (grid.y > 1) {
+        const int64_t rows = nt * H;
+        hipLaunchKernelGGL((window_attn_combine_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(DV < 256 ? 64 : 256), 0, s,
+                           out, po, pml, rows, DV, static_cast<int>(grid.y));
+    }
     return check_launch();
 }
 
@@ -248,9 +330,11 @@ extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cac
                                      const int32_t *tile_row0, const int32_t *tile_cnt, const float *talk,
                                      int32_t num_tiles, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
                                      int32_t vdim, int64_t q_tok_stride, int32_t window, float scale, float softcap,
-                                     int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
-                                     swl_stream_t stream) {
-    if (num_tiles < 0 || window < 0) return SWL_ERR_BAD_ARG;
+                                     int32_t max_blocks_per_seq, int64_t block_stride, int32_t key_splits,
+                                     float *scratch, int64_t num_tokens, int32_t dtype, swl_stream_t stream) {
+    if (num_tiles < 0 || window < 0 || key_splits < 1 || key_splits > 64) return SWL_ERR_BAD_ARG;
+    if (key_splits > 1 && (!scratch || num_tokens <= 0 || (reinterpret_cast<uintptr_t>(scratch) & 15)))
+        return SWL_ERR_BAD_ARG;
     if (!swl_window_attn_tiles_supported(num_q_heads, num_kv_heads, dim, vdim, dtype)) return SWL_ERR_UNSUPPORTED;
     if (num_tiles == 0) return SWL_OK;
     if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !tile_row0 || !tile_cnt || !talk)
@@ -261,14 +345,18 @@ extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cac
     int hpw = (num_q_heads + swl::kWmWaves - 1) / swl::kWmWaves;
     hpw = hpw <= 1 ? 1 : hpw <= 2 ? 2 : hpw <= 4 ? 4 : 8;
     const size_t lds = static_cast<size_t>(num_q_heads) * 64 * 4 * sizeof(float);
-    const dim3 grid(static_cast<unsigned>(num_tiles));
+    const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(key_splits));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // scratch: [splits][tokens][H][vdim] fp32 partial outputs, then [splits][tokens][H][2] (maximum, sum)
+    float *part_o = scratch;
+    float *part_ml = scratch ? scratch + static_cast<int64_t>(key_splits) * num_tokens * num_q_heads * vdim : nullptr;
 #define SWL_WM_SHAPE(DD, DDV)                                                                                             \
     if (dim == DD && vdim == DDV)                                                                                         \
         return swl::launch_wm<T, DD, DDV>(hpw, grid, lds, s, static_cast<T *>(out), static_cast<const T *>(q),           \
                                           static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, \
                                           tok_seq, tok_pos, tile_row0, tile_cnt, talk, num_q_heads, num_kv_heads,        \
-                                          q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride);
+                                          q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride, part_o, \
+                                          part_ml, num_tokens);
     SWL_DISPATCH_DTYPE(dtype, T, {
         SWL_WM_SHAPE(64, 64)
         SWL_WM_SHAPE(128, 128)

@@ -110,7 +110,7 @@ class KekapelModel:
         for run in cfg.layer_runs:
             lcfg, lw = cfg.layers[run.layer], self.weight.layers[run.layer]
             s = _Sublayer()
-            s.kind, s.run, s.op = "mixer", run.index, KekapelAttention(lcfg, lw, eps, skinny)
+            s.kind, s.run, s.op = "mixer", run.index, KekapelAttention(lcfg, lw, eps, skinny, cfg.max_position_embeddings)
             s.pre, s.post, s.pass_index = (lw.norm1_w, lw.norm1_b), (lw.norm1b_w, lw.norm1b_b), run.pass_index
             s.ends_run = lcfg.mlp is None
             self.sublayers.append(s)

@@ -19,6 +19,46 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top_k: 
     return idx, wts
 
 
+# From this many assignments per expert on (on average), a step's expert products are library GEMMs over the assignments
+# sorted by expert; below, every assignment streams its expert's rows (decode batches: capturable, no host read-back).
+GROUPED_MIN_ROWS_PER_EXPERT = 16
+
+
+def moe_experts_grouped(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
+                        limit: float) -> torch.Tensor:
+    """The same function as moe_experts for steps with many tokens: assignments sorted by expert (stable), one [rows, width]
+    x [width, 2 ff] and one [rows, ff] x [ff, width] library product per expert that received tokens, the activation and
+    the weighted combination as kernels. Reads the per-expert counts back to the host (one sync per call)."""
+    n, width = h.shape
+    experts, two_ff, _ = gate_up.shape
+    ff, top_k = two_ff // 2, idx.shape[1]
+    flat = idx.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)                # sorted position -> assignment (token * top + j)
+    counts = torch.bincount(flat, minlength=experts).tolist()
+    where = torch.empty_like(order)
+    where[order] = torch.arange(order.numel(), device=order.device)     # assignment -> sorted position
+    xs = h.index_select(0, order // top_k)
+    code, stream = _hip.dtype_code3(h.dtype), _hip.stream()
+    gu = torch.empty((n * top_k, two_ff), dtype=h.dtype, device=h.device)
+    off = 0
+    for e, c in enumerate(counts):
+        if c:
+            torch.mm(xs[off:off + c], gate_up[e].t(), out=gu[off:off + c])
+            off += c
+    y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
+    _hip.call("swl_glu_clamp", _hip.ptr(y), _hip.ptr(gu), n * top_k, ff, float(limit), code, stream)
+    rows = torch.empty((n * top_k, width), dtype=h.dtype, device=h.device)
+    off = 0
+    for e, c in enumerate(counts):
+        if c:
+            torch.mm(y[off:off + c], down[e].t(), out=rows[off:off + c])
+            off += c
+    out = torch.empty((n, width), dtype=h.dtype, device=h.device)
+    _hip.call("swl_moe_combine", _hip.ptr(out), _hip.ptr(rows), _hip.ptr(where), _hip.ptr(wts), n, width, top_k, code,
+              stream)
+    return out
+
+
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
                 limit: float) -> torch.Tensor:
     """-> [T, width]: sum_j wts[t, j] * expert idx[t, j] applied to h[t]. gate_up [experts, 2 ff, width], down
@@ -28,6 +68,8 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: 
     ff, top_k = two_ff // 2, idx.shape[1]
     assert gate_up.is_contiguous() and down.is_contiguous() and down.shape == (experts, width, ff)
     assert gate_up.dtype == down.dtype == h.dtype and idx.dtype == torch.int32 and wts.dtype == torch.float32
+    if n * top_k >= GROUPED_MIN_ROWS_PER_EXPERT * experts and not torch.cuda.is_current_stream_capturing():
+        return moe_experts_grouped(h, idx, wts, gate_up, down, limit)
     code, stream = _hip.dtype_code3(h.dtype), _hip.stream()
     y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
     _hip.call("swl_moe_gate_up", _hip.ptr(y), _hip.ptr(h), _hip.ptr(gate_up), _hip.ptr(idx), n, width, ff, top_k,

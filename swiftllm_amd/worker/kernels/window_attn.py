@@ -39,9 +39,31 @@ def qknorm_and_store_kv(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: torch.T
               _hip.dtype_code3(qkv.dtype), _hip.stream())
 
 
-# Steps with at least this many tokens go to the matrix-core kernel (tiles of 16 queries); smaller ones — decode batches — to
-# the per-token kernel, whose workgroups are not mostly padding there.
-TILES_MIN_TOKENS = 48
+# Steps with at least this many tokens go to the matrix-core kernel (tiles of up to 16 queries; a decoded token is a tile of
+# one: the matrix core is mostly padding there, but the kernel reads every page once with wide loads and shares a tile's pages
+# out over several workgroups when there are few tiles).
+TILES_MIN_TOKENS = 1
+_NUM_CUS = 256
+_scratch = {}       # device -> persistent fp32 scratch of the key-split partials (fixed address: hipGraph replays use it)
+_retired = []
+
+
+def _split_scratch(device, floats: int) -> torch.Tensor:
+    buf = _scratch.get(device)
+    if buf is None or buf.numel() < floats:
+        if buf is not None:
+            _retired.append(buf)        # a captured graph may still replay against it
+        buf = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=device)
+        _scratch[device] = buf
+    return buf
+
+
+def choose_key_splits(num_tiles: int, mixer, max_positions: int) -> int:
+    """Workgroups per tile: enough to occupy the chip when a step has few tiles, never more than the pages a tile can see.
+    A function of the tile count and the model only (not of positions), so a captured decode graph stays valid."""
+    span = mixer.window if mixer.window > 0 else max_positions
+    pages = span // 16 + 2
+    return max(1, min(_NUM_CUS // max(num_tiles, 1), pages // 4, 16))
 
 
 def tiles_supported(mixer, dtype: torch.dtype) -> bool:
@@ -53,7 +75,7 @@ def tiles_supported(mixer, dtype: torch.dtype) -> bool:
 
 def window_attention(qkv: torch.Tensor, talk: torch.Tensor, pool: torch.Tensor, pool_slice: PoolSlice,
                      block_table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, mixer,
-                     tiles=None) -> torch.Tensor:
+                     tiles=None, max_positions: int = 1 << 20) -> torch.Tensor:
     """-> [T, heads * vdim]. The queries are the (already normalised) first columns of qkv; keys and values come from the
     pool, which already holds this step's tokens. `tiles` = (tile_row0, tile_cnt) device arrays: the step cut into runs of
     up to 16 consecutive tokens of one sequence — given, and the shape served, the matrix-core kernel runs."""
@@ -65,11 +87,16 @@ def window_attention(qkv: torch.Tensor, talk: torch.Tensor, pool: torch.Tensor, 
     esize = pool.element_size()
     if tiles is not None and n >= TILES_MIN_TOKENS and tiles_supported(mixer, qkv.dtype):
         row0, cnt = tiles
+        splits = choose_key_splits(row0.shape[0], mixer, max_positions)
+        scratch = None
+        if splits > 1:
+            scratch = _split_scratch(qkv.device, splits * n * mixer.num_q_heads * (mixer.value_dim + 2))
         _hip.call("swl_window_attn_tiles", _hip.ptr(out), _hip.ptr(qkv), pool.data_ptr() + pool_slice.k_offset * esize,
                   pool.data_ptr() + pool_slice.v_offset * esize, _hip.ptr(block_table), _hip.ptr(tok_seq),
                   _hip.ptr(tok_pos), _hip.ptr(row0), _hip.ptr(cnt), _hip.ptr(talk), row0.shape[0], mixer.num_q_heads,
                   mixer.num_kv_heads, mixer.head_dim, mixer.value_dim, qkv.stride(0), mixer.window, float(mixer.scale),
-                  float(mixer.softcap), block_table.shape[1], pool.shape[1], _hip.dtype_code(qkv.dtype), _hip.stream())
+                  float(mixer.softcap), block_table.shape[1], pool.shape[1], splits, _hip.ptr(scratch), n,
+                  _hip.dtype_code(qkv.dtype), _hip.stream())
         return out
     _hip.call("swl_window_attn", _hip.ptr(out), _hip.ptr(qkv), pool.data_ptr() + pool_slice.k_offset * esize,
               pool.data_ptr() + pool_slice.v_offset * esize, _hip.ptr(block_table), _hip.ptr(tok_seq), _hip.ptr(tok_pos),

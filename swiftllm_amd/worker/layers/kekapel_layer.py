@@ -20,8 +20,9 @@ class KekapelAttention:
     """q/k/v projection -> per-head q/k norm + KV store -> windowed, capped, head-mixed attention over the pool -> output
     projection."""
 
-    def __init__(self, layer_config, weight, eps: float, skinny: bool):
+    def __init__(self, layer_config, weight, eps: float, skinny: bool, max_positions: int = 1 << 20):
         self.mixer, self.w, self.eps, self.skinny = layer_config.mixer, weight, eps, skinny
+        self.max_positions = max_positions
 
     def forward(self, h: torch.Tensor, pool, pool_slice, block_table, tok_seq, tok_pos, tiles=None) -> torch.Tensor:
         qkv = _project(h, self.w.qkv, self.skinny)
@@ -30,7 +31,8 @@ class KekapelAttention:
         if pool is None:    # memory profiling: the attention's output buffer without its reads
             attn = torch.zeros((h.shape[0], self.mixer.num_q_heads * self.mixer.value_dim), dtype=h.dtype, device=h.device)
         else:
-            attn = window_attention(qkv, self.w.talk, pool, pool_slice, block_table, tok_seq, tok_pos, self.mixer, tiles)
+            attn = window_attention(qkv, self.w.talk, pool, pool_slice, block_table, tok_seq, tok_pos, self.mixer, tiles,
+                                    self.max_positions)
         return _project(attn, self.w.o, self.skinny)
 
 

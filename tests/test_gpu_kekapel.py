@@ -100,11 +100,14 @@ def test_polynorm(dtype):
     assert (got - want).abs().max() < (1e-5 if dtype == torch.float32 else 3e-2)
 
 
+@pytest.mark.parametrize("n", [23, 300])       # per-assignment kernels / assignments sorted by expert + library products
 @pytest.mark.parametrize("experts,top", [(5, 2), (70, 4), (3, 3), (4, 1)])
-def test_moe_router_and_experts(experts, top):
+def test_moe_router_and_experts(experts, top, n):
+    from swiftllm_amd.worker.kernels import moe
     from swiftllm_amd.worker.kernels.moe import moe_experts, moe_route
     g = torch.Generator().manual_seed(experts)
-    n, w, ff, limit = 23, 40, 24, 0.9
+    w, ff, limit = 40, 24, 0.9
+    assert (300 * 2 >= moe.GROUPED_MIN_ROWS_PER_EXPERT * 5) and (23 * 2 < moe.GROUPED_MIN_ROWS_PER_EXPERT * 5)   # both paths run
     h = torch.randn(n, w, generator=g)
     W = {"router": torch.randn(experts, w, generator=g), "router.b": torch.randn(experts, generator=g)}
     for e in range(experts):
