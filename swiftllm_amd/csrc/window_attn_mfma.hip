@@ -22,31 +22,20 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
 // D[16x16] += A[16x16] B[16x16]; lane l holds A[l % 16][4 (l / 16) + 0..3], B[4 (l / 16) + 0..3][l % 16], D[4 (l / 16) + 0..3][l % 16]
-__device__ __forceinline__ float4_t mfma16(const bf16 (&a)[4], const bf16 (&b)[4], float4_t c) {
-    short4v av, bv;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        av[i] = __builtin_bit_cast(short, a[i]);
-        bv[i] = __builtin_bit_cast(short, b[i]);
-    }
-    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av, bv, c, 0, 0, 0);
+// (operand fragments stay packed 64-bit vectors from the load to the matrix core: no per-element repacking)
+template <typename T>
+using vec4_t = T __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float4_t mfma16(vec4_t<bf16> a, vec4_t<bf16> b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, a), __builtin_bit_cast(short4v, b), c, 0, 0, 0);
 }
-__device__ __forceinline__ float4_t mfma16(const f16 (&a)[4], const f16 (&b)[4], float4_t c) {
-    half4v av, bv;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        av[i] = a[i];
-        bv[i] = b[i];
-    }
-    return __builtin_amdgcn_mfma_f32_16x16x16f16(av, bv, c, 0, 0, 0);
+__device__ __forceinline__ float4_t mfma16(vec4_t<f16> a, vec4_t<f16> b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4v, a), __builtin_bit_cast(half4v, b), c, 0, 0, 0);
 }
 
 template <typename T>
-__device__ __forceinline__ void load4(T (&dst)[4], const T *p) {    // 8-byte load
-    typedef T vec4 __attribute__((ext_vector_type(4)));
-    const vec4 v = *reinterpret_cast<const vec4 *>(p);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) dst[i] = v[i];
+__device__ __forceinline__ void load4(vec4_t<T> &dst, const T *p) {    // 8-byte load
+    dst = *reinterpret_cast<const vec4_t<T> *>(p);
 }
 
 __device__ __forceinline__ float fast_tanh(float x) {
@@ -60,16 +49,22 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk, int H, int G,
     int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
-    float *part_o, float *part_ml, int64_t num_tokens) {
-    extern __shared__ float s_lds[];    // [H][64 lanes][4]
+    float *part_o, float *part_ml, int64_t num_tokens, int nbuf) {
+    // [nbuf][H][64 lanes][4] capped scores of a page, then [H][H] the mixing matrix. nbuf = 2: pages alternate between two
+    // score buffers and ONE barrier per page suffices (a wave that is a page ahead writes the other buffer)
+    extern __shared__ float s_all[];
+    float *tk = s_all + nbuf * H * 256;
     constexpr int CT = DV / 16;         // 16-column tiles of the value head
     constexpr float kLog2e = 1.4426950408889634f;
     const int tile = blockIdx.x;
-    const int row0 = tile_row0[tile], cnt = tile_cnt[tile];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int row0 = __builtin_amdgcn_readfirstlane(tile_row0[tile]), cnt = __builtin_amdgcn_readfirstlane(tile_cnt[tile]);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // (tells the compiler that it is wave-uniform)
     const int li = lane & 15, lq = lane >> 4;       // query (or operand row) index; quarter
-    const int p0 = tok_pos[row0];
-    const int32_t *bt = block_table + static_cast<int64_t>(tok_seq[row0]) * max_blocks_per_seq;
+    for (int i = tid; i < H * H; i += kWmThreads) tk[i] = talk[i];
+    __syncthreads();
+    const int p0 = __builtin_amdgcn_readfirstlane(tok_pos[row0]);
+    const int32_t *bt = block_table + static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tok_seq[row0])) * max_blocks_per_seq;
     const int rep = H / G;
     const int h0 = wave * HPW;
     const int qpos = p0 + li;                        // this lane's query position (meaningful when li < cnt)
@@ -98,9 +93,9 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
     // page's mix / softmax / value products run; the value fragments of a page are requested before its score products.
     constexpr int KS = D / 16;
     constexpr bool PIPE = HPW * D <= 512 && HPW * DV <= 512;
-    T qf[PIPE ? HPW : 1][KS][4], kf[PIPE ? HPW : 1][KS][4];
-    auto fetch_k = [&](int kb) {
-        const T *kblk = k_cache + static_cast<int64_t>(bt[kb]) * block_stride;
+    vec4_t<T> qf[PIPE ? HPW : 1][KS], kf[PIPE ? HPW : 1][KS];
+    auto fetch_k = [&](int64_t blk) {
+        const T *kblk = k_cache + blk * block_stride;
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int g = min(h0 + hh, H - 1);
@@ -116,16 +111,21 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
 #pragma unroll
             for (int e = 0; e < KS; ++e) load4(qf[hh][e], qrow + g * D + 4 * lq + e * 16);     // B: query li
         }
-        if (kb0 <= kb1) fetch_k(kb0);
+    }
+    int blk_next = kb0 <= kb1 ? __builtin_amdgcn_readfirstlane(bt[kb0]) : 0;
+    if constexpr (PIPE) {
+        if (kb0 <= kb1) fetch_k(blk_next);
     }
 
     for (int kb = kb0; kb <= kb1; ++kb) {
-        const int64_t blk = bt[kb];
+        float *s_lds = s_all + (nbuf == 2 && ((kb - kb0) & 1) ? H * 256 : 0);
+        const int64_t blk = blk_next;
+        const int nxt = kb < kb1 ? bt[kb + 1] : 0;      // the next page's block id, requested a page ahead of its use
         const T *kblk = k_cache + blk * block_stride;
         const T *vblk = v_cache + blk * block_stride;
         // value fragments of this page, A operand of O^T += V^T P^T: V^T[col ct * 16 + li][keys 4 lq .. 4 lq + 3] — the pool keeps
         // a page's values transposed ([kv head][column][16 keys]), so this is one 8-byte load
-        T vfrag[PIPE ? HPW : 1][CT][4];
+        vec4_t<T> vfrag[PIPE ? HPW : 1][CT];
         auto fetch_v = [&](int hh) {
             const int kv = min(h0 + hh, H - 1) / rep;
 #pragma unroll
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
                     const T *qr = qrow + g * D + 4 * lq;
 #pragma unroll
                     for (int e = 0; e < KS; ++e) {
-                        T a[4], b[4];
+                        vec4_t<T> a, b;
                         load4(a, kr + e * 16);
                         load4(b, qr + e * 16);
                         st = mfma16(a, b, st);
@@ -168,8 +168,9 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
             }
         }
         __syncthreads();
+        blk_next = __builtin_amdgcn_readfirstlane(nxt);
         if constexpr (PIPE) {
-            if (kb < kb1) fetch_k(kb + 1);
+            if (kb < kb1) fetch_k(blk_next);
         }
         // ---- 2. mix, mask, online softmax; 3. O^T += V^T P^T for this wave's heads ------------------------------------------
         const int kpos0 = kb * kWmTile + 4 * lq;     // position of this lane's key r = 0
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
 #pragma unroll
             for (int hh = 0; hh < HPW; ++hh) {
                 const int h = min(h0 + hh, H - 1);
-                const float tw = talk[h * H + g];       // wave-uniform address: a scalar load
+                const float tw = tk[h * H + g];         // wave-uniform address: an LDS broadcast
 #pragma unroll
                 for (int r = 0; r < 4; ++r) mixed[hh][r] += tw * sv[r];
             }
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
                 const float mnew = fmaxf(mrun[hh], cmax);
                 const float alpha = fast_exp2((mrun[hh] - mnew) * kLog2e);
                 mrun[hh] = mnew;
-                T phi[4], plo[4];
+                vec4_t<T> phi, plo;
                 float psum = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
                 }
             }
         }
-        __syncthreads();    // every wave is done with this page's scores before the next page overwrites them
+        if (nbuf == 1) __syncthreads();     // every wave is done with this page's scores before the next page overwrites them
     }
     // ---- epilogue: O[query li][h][ct * 16 + 4 lq + r] = O^T / l -------------------------------------------------------------------
 #pragma unroll
@@ -294,10 +295,10 @@ template <typename T, int D, int DV>
 int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q, const T *kc, const T *vc,
               const int32_t *bt, const int32_t *ts, const int32_t *tp, const int32_t *r0, const int32_t *cn,
               const float *talk, int H, int G, int64_t qs, int window, float scale, float softcap, int mb, int64_t bs,
-              float *po, float *pml, int64_t nt) {
+              float *po, float *pml, int64_t nt, int nbuf) {
 #define SWL_WM_LAUNCH(HPW)                                                                                              \
     hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW>), grid, dim3(kWmThreads), lds, s, out, q, kc, vc, bt, ts, \
-                       tp, r0, cn, talk, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt)
+                       tp, r0, cn, talk, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf)
     switch (hpw) {
     case 1: SWL_WM_LAUNCH(1); break;
     case 2: SWL_WM_LAUNCH(2); break;
@@ -344,7 +345,9 @@ extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cac
         return SWL_ERR_BAD_ARG;     // 8-byte operand loads
     int hpw = (num_q_heads + swl::kWmWaves - 1) / swl::kWmWaves;
     hpw = hpw <= 1 ? 1 : hpw <= 2 ? 2 : hpw <= 4 ? 4 : 8;
-    const size_t lds = static_cast<size_t>(num_q_heads) * 64 * 4 * sizeof(float);
+    const size_t one = static_cast<size_t>(num_q_heads) * 256, mixw = static_cast<size_t>(num_q_heads) * num_q_heads;
+    const int nbuf = (2 * one + mixw) * sizeof(float) <= 64 * 1024 ? 2 : 1;
+    const size_t lds = (nbuf * one + mixw) * sizeof(float);
     const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(key_splits));
     hipStream_t s = static_cast<hipStream_t>(stream);
     // scratch: [splits][tokens][H][vdim] fp32 partial outputs, then [splits][tokens][H][2] (maximum, sum)
@@ -356,7 +359,7 @@ extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cac
                                           static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, \
                                           tok_seq, tok_pos, tile_row0, tile_cnt, talk, num_q_heads, num_kv_heads,        \
                                           q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride, part_o, \
-                                          part_ml, num_tokens);
+                                          part_ml, num_tokens, nbuf);
     SWL_DISPATCH_DTYPE(dtype, T, {
         SWL_WM_SHAPE(64, 64)
         SWL_WM_SHAPE(128, 128)
