@@ -557,6 +557,13 @@ int swl_moe_gate_up(void *y, const void *h, const void *gate_up, const int32_t *
 /* Large steps (prompt portions): assignments are sorted by expert and every expert's rows go through the library GEMM;
  * swl_glu_clamp: y[r][f] = act of [gate | up] product rows gate_up[r][2 ff]; swl_moe_combine: out[t] = sum_j w[t][j] *
  * rows[where[t * top + j]] (fp32, fixed order). dtype may be SWL_F32. */
+/* Decode-sized steps, 16-bit, on the matrix core: a workgroup per (expert, 64 outputs) loads every weight fragment once and
+ * multiplies it with all assignments of the expert (an expert's weights are streamed once per step). glu = 1: out = y[T * top, ff] from x = h[T, width]
+ * and w = gate_up; glu = 0: out = rows[T * top, width] (plain products, for swl_moe_combine) from x = y and w = down. */
+int swl_moe_expert_stationary_supported(int64_t num_tokens, int32_t width, int32_t ff, int32_t top, int32_t dtype);
+int swl_moe_expert_stationary(void *out, const void *x, const void *w, const int32_t *expert_idx, int64_t num_tokens,
+                              int32_t experts, int32_t width, int32_t ff, int32_t top, int32_t glu, float limit,
+                              int32_t dtype, swl_stream_t stream);
 int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t dtype,
                   swl_stream_t stream);
 int swl_moe_combine(void *out, const void *rows, const int64_t *where, const float *expert_w, int64_t num_tokens,

@@ -105,6 +105,7 @@ SIGNATURES = {
     "swl_polynorm": [_P, _P, _F32, _F32, _F32, _F32, _F32, _I64, _I32, _I32, _P],
     "swl_moe_route": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
     "swl_moe_gate_up": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _P],
+    "swl_moe_expert_stationary": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I32, _F32, _I32, _P],
     "swl_glu_clamp": [_P, _P, _I64, _I32, _F32, _I32, _P],
     "swl_moe_combine": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _P],
     "swl_moe_down_combine": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
@@ -123,6 +124,7 @@ _SPECIAL = {
     "swl_gemm_packed_wide_choose_splits": ([_I32, _I32, _I32], _I32),
     "swl_gemm_tiny_max_tokens": ([], _I32),
     "swl_gemm_rows_supported": ([_I32, _I32, _I32], _I32),
+    "swl_moe_expert_stationary_supported": ([_I64, _I32, _I32, _I32, _I32], _I32),
     "swl_window_attn_tiles_supported": ([_I32, _I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_supported": ([_I32, _I32, _I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_slots_per_layer": ([_I32, _I32, _I32, _I32], _I32),

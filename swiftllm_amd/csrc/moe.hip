@@ -161,6 +161,92 @@ __global__ __launch_bounds__(kMoeThreads) void moe_down_combine_kernel(T *out, c
     }
 }
 
+
+// ---- expert-stationary products for decode-sized steps -----------------------------------------------------------------------
+// out[a][n] = sum_k W[e][n][k] X[xrow(a)][k] for the assignments a of expert e, on the matrix core. A workgroup owns (expert,
+// 64 outputs n), a wave 16 of them: per 16-wide k step it loads its weight fragment ONCE (A operand: row n, 8 bytes per lane)
+// and multiplies it with the input fragments of up to four tiles of 16 assignments (B operand: the assignment's input row,
+// read through the caches — the rows of a decode step are few and stay resident). An expert's weights are thus streamed once
+// per step however many tokens chose it (the per-assignment kernels above stream them once per token). GLU: n indexes ff,
+// the gate row n and the up row ff + n share the input fragments and meet in the clamped gated unit; X rows are tokens
+// (a / top). Otherwise (down projection) X rows are assignments and the output is the plain product, rounded to T.
+constexpr int kEsRows = 64;         // outputs per workgroup (16 per wave)
+constexpr int kEsTiles = 4;         // tiles of 16 assignments per pass over the weights
+constexpr int kEsMaxAssign = 1024;  // assignments per step (the sorted library path serves larger steps)
+
+template <typename T, bool GLU>
+__global__ __launch_bounds__(kMoeThreads) void moe_expert_stationary_kernel(T *out, const T *x, const T *w,
+                                                                            const int32_t *expert_idx, int assignments,
+                                                                            int K, int N, int top, float limit) {
+    __shared__ int mine[kEsMaxAssign];
+    __shared__ int count;
+    const int e = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int li = lane & 15, lq = lane >> 4;
+    if (threadIdx.x == 0) count = 0;
+    __syncthreads();
+    for (int a = threadIdx.x; a < assignments; a += kMoeThreads)
+        if (expert_idx[a] == e) mine[atomicAdd(&count, 1)] = a;
+    __syncthreads();
+    const int m = count;
+    const int n0 = blockIdx.y * kEsRows + wave * 16;
+    if (m == 0 || n0 >= N) return;
+    const int nrow = min(n0 + li, N - 1);       // (rows past N compute a duplicate that is never stored)
+    const T *wg = w + (static_cast<int64_t>(e) * (GLU ? 2 : 1) * N + nrow) * K + 4 * lq;
+    const T *wu = wg + static_cast<int64_t>(N) * K;
+    for (int pass = 0; pass < m; pass += 16 * kEsTiles) {
+        const int ntile = min(kEsTiles, (m - pass + 15) / 16);
+        int arow[kEsTiles];
+        const T *xp[kEsTiles];
+#pragma unroll
+        for (int t = 0; t < kEsTiles; ++t) {
+            const int i = pass + t * 16 + li;
+            const int a = i < m ? mine[i] : -1;
+            arow[t] = a;
+            xp[t] = x + static_cast<int64_t>(a < 0 ? 0 : (GLU ? a / top : a)) * K + 4 * lq;
+        }
+        float4_t accg[kEsTiles], accu[kEsTiles];
+#pragma unroll
+        for (int t = 0; t < kEsTiles; ++t) accg[t] = accu[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+        for (int k0 = 0; k0 < K; k0 += 16) {
+            vec4_t<T> ag, au;
+            load4(ag, wg + k0);
+            if constexpr (GLU) load4(au, wu + k0);
+#pragma unroll
+            for (int t = 0; t < kEsTiles; ++t) {
+                if (t < ntile) {
+                    vec4_t<T> b = vec4_t<T>{};
+                    if (arow[t] >= 0) load4(b, xp[t] + k0);
+                    accg[t] = mfma16(ag, b, accg[t]);
+                    if constexpr (GLU) accu[t] = mfma16(au, b, accu[t]);
+                }
+            }
+        }
+        // accumulator r of lane (li, lq): output row n0 + 4 lq + r of the assignment in column li
+#pragma unroll
+        for (int t = 0; t < kEsTiles; ++t) {
+            mfma_results_tie(accg[t]);
+            mfma_results_ready<4>(accu[t]);
+            if (t < ntile && arow[t] >= 0) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n0 + 4 * lq + r;
+                    if (n < N) {
+                        float v = accg[t][r];
+                        if constexpr (GLU) {
+                            const float g = fminf(v, limit);
+                            const float u = fminf(fmaxf(accu[t][r], -limit), limit);
+                            v = g * (1.0f / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
+                        }
+                        out[static_cast<int64_t>(arow[t]) * N + n] = to_t<T>(v);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // y[r][f] = act(gu[r][f], gu[r][ff + f]) for rows of [gate | up] products that came from a library GEMM
 template <typename T>
 __global__ __launch_bounds__(kMoeThreads) void glu_clamp_kernel(T *y, const T *gu, int64_t total, int ff, float limit) {
@@ -187,6 +273,40 @@ __global__ __launch_bounds__(kMoeThreads) void moe_combine_kernel(T *out, const 
 }
 
 } // namespace swl
+
+/* 1 when swl_moe_expert_stationary serves the shape: 16-bit, both reduction lengths multiples of 16, at most 1024
+ * assignments. */
+extern "C" int swl_moe_expert_stationary_supported(int64_t num_tokens, int32_t width, int32_t ff, int32_t top, int32_t dtype) {
+    if (dtype != SWL_F16 && dtype != SWL_BF16) return 0;
+    if (width <= 0 || ff <= 0 || (width & 15) || (ff & 15)) return 0;
+    return num_tokens * top <= swl::kEsMaxAssign;
+}
+
+extern "C" int swl_moe_expert_stationary(void *out, const void *x, const void *w, const int32_t *expert_idx,
+                                         int64_t num_tokens, int32_t experts, int32_t width, int32_t ff, int32_t top,
+                                         int32_t glu, float limit, int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || experts <= 0 || top <= 0) return SWL_ERR_BAD_ARG;
+    if (!swl_moe_expert_stationary_supported(num_tokens, width, ff, top, dtype)) return SWL_ERR_UNSUPPORTED;
+    if (num_tokens == 0) return SWL_OK;
+    if (!out || !x || !w || !expert_idx || !swl::aligned16(x) || !swl::aligned16(w)) return SWL_ERR_BAD_ARG;
+    const int K = glu ? width : ff, N = glu ? ff : width;
+    const int assignments = static_cast<int>(num_tokens * top);
+    const size_t lds = 0;
+    const dim3 grid(static_cast<unsigned>(experts), static_cast<unsigned>((N + swl::kEsRows - 1) / swl::kEsRows));
+    if (grid.y > 65535) return SWL_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    SWL_DISPATCH_DTYPE(dtype, T, {
+        if (glu)
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, true>), grid, dim3(swl::kMoeThreads), lds, s,
+                               static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
+                               assignments, K, N, top, limit);
+        else
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, false>), grid, dim3(swl::kMoeThreads), lds, s,
+                               static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
+                               assignments, K, N, top, limit);
+    });
+    return swl::check_launch();
+}
 
 extern "C" int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t dtype,
                              swl_stream_t stream) {

@@ -260,6 +260,28 @@ __device__ __forceinline__ void mfma_results_ready(V &acc) {
     else asm volatile("s_nop 15" : "+v"(acc));                                 // 16 wait states
 }
 
+// ---- 16x16x16 matrix-core step on packed 64-bit operand fragments ------------------------------------------------------
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+// D[16x16] += A[16x16] B[16x16]; lane l holds A[l % 16][4 (l / 16) + 0..3], B[4 (l / 16) + 0..3][l % 16], D[4 (l / 16) + 0..3][l % 16]
+// (operand fragments stay packed 64-bit vectors from the load to the matrix core: no per-element repacking)
+template <typename T>
+using vec4_t = T __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float4_t mfma16(vec4_t<bf16> a, vec4_t<bf16> b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, a), __builtin_bit_cast(short4v, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ float4_t mfma16(vec4_t<f16> a, vec4_t<f16> b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4v, a), __builtin_bit_cast(half4v, b), c, 0, 0, 0);
+}
+
+template <typename T>
+__device__ __forceinline__ void load4(vec4_t<T> &dst, const T *p) {    // 8-byte load
+    dst = *reinterpret_cast<const vec4_t<T> *>(p);
+}
+
+
 // exp2 on the hardware transcendental unit (v_exp_f32 IS 2^x).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

@@ -1,7 +1,7 @@
 // window_attn_mfma.hip — the matrix-core form of window_attn.hip for 16-bit storage: tiles of up to 16 consecutive query
 // tokens of one sequence against 16-key pages of the pool.
 //
-// One workgroup (4 waves) per query tile. The head mix couples all heads of a (query, key) pair, so the heads are split
+// One workgroup (4 waves; 8 for more than 16 heads) per query tile. The head mix couples all heads of a (query, key) pair, so the heads are split
 // over the waves: wave w owns heads [w * HPW, (w + 1) * HPW) for the score products AND for the outputs, and the capped
 // scores of all heads meet in LDS in between. Per 16-key page:
 //   1. S^T_g = K_kv(g) Q_g^T      (16 keys x 16 queries, MFMA 16x16x16, fp32 accumulate), scale, tanh cap -> LDS [H][256] fp32
@@ -18,34 +18,14 @@ constexpr int kWmThreads = 256;
 constexpr int kWmWaves = 4;
 constexpr int kWmTile = 16;     // queries per tile = keys per page = MFMA edge
 
-typedef short short4v __attribute__((ext_vector_type(4)));
-typedef _Float16 half4v __attribute__((ext_vector_type(4)));
-
-// D[16x16] += A[16x16] B[16x16]; lane l holds A[l % 16][4 (l / 16) + 0..3], B[4 (l / 16) + 0..3][l % 16], D[4 (l / 16) + 0..3][l % 16]
-// (operand fragments stay packed 64-bit vectors from the load to the matrix core: no per-element repacking)
-template <typename T>
-using vec4_t = T __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ float4_t mfma16(vec4_t<bf16> a, vec4_t<bf16> b, float4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, a), __builtin_bit_cast(short4v, b), c, 0, 0, 0);
-}
-__device__ __forceinline__ float4_t mfma16(vec4_t<f16> a, vec4_t<f16> b, float4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4v, a), __builtin_bit_cast(half4v, b), c, 0, 0, 0);
-}
-
-template <typename T>
-__device__ __forceinline__ void load4(vec4_t<T> &dst, const T *p) {    // 8-byte load
-    dst = *reinterpret_cast<const vec4_t<T> *>(p);
-}
-
 __device__ __forceinline__ float fast_tanh(float x) {
     // 1 - 2 / (e^{2x} + 1); exp2 overflow to inf gives exactly 1, underflow to 0 gives exactly -1
     const float e = fast_exp2(x * 2.885390081777927f);
     return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 
-template <typename T, int D, int DV, int HPW>
-__global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
+template <typename T, int D, int DV, int HPW, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk, int H, int G,
     int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
@@ -61,7 +41,7 @@ __global__ __launch_bounds__(kWmThreads, 1) void window_attn_mfma_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // (tells the compiler that it is wave-uniform)
     const int li = lane & 15, lq = lane >> 4;       // query (or operand row) index; quarter
-    for (int i = tid; i < H * H; i += kWmThreads) tk[i] = talk[i];
+    for (int i = tid; i < H * H; i += NW * 64) tk[i] = talk[i];
     __syncthreads();
     const int p0 = __builtin_amdgcn_readfirstlane(tok_pos[row0]);
     const int32_t *bt = block_table + static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tok_seq[row0])) * max_blocks_per_seq;
@@ -296,14 +276,16 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
               const int32_t *bt, const int32_t *ts, const int32_t *tp, const int32_t *r0, const int32_t *cn,
               const float *talk, int H, int G, int64_t qs, int window, float scale, float softcap, int mb, int64_t bs,
               float *po, float *pml, int64_t nt, int nbuf) {
-#define SWL_WM_LAUNCH(HPW)                                                                                              \
-    hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW>), grid, dim3(kWmThreads), lds, s, out, q, kc, vc, bt, ts, \
+#define SWL_WM_LAUNCH(HPW, NW)                                                                                          \
+    hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW, NW>), grid, dim3(NW * 64), lds, s, out, q, kc, vc, bt, ts, \
                        tp, r0, cn, talk, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf)
+    // heads per wave x waves: up to 16 heads on four waves, more on eight (four heads per wave at most: the accumulators of
+    // eight 128-wide heads do not fit a wave's registers)
     switch (hpw) {
-    case 1: SWL_WM_LAUNCH(1); break;
-    case 2: SWL_WM_LAUNCH(2); break;
-    case 4: SWL_WM_LAUNCH(4); break;
-    case 8: SWL_WM_LAUNCH(8); break;
+    case 1: SWL_WM_LAUNCH(1, 4); break;
+    case 2: SWL_WM_LAUNCH(2, 4); break;
+    case 4: SWL_WM_LAUNCH(4, 4); break;
+    case 8: SWL_WM_LAUNCH(4, 8); break;
     default: return SWL_ERR_UNSUPPORTED;
     }
 #undef SWL_WM_LAUNCH

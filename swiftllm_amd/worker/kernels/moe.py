@@ -24,6 +24,18 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top_k: 
 GROUPED_MIN_ROWS_PER_EXPERT = 16
 
 
+_identities = {}
+
+
+def _identity(n: int, device) -> torch.Tensor:
+    """arange(n) int64 on the device, kept (a captured graph reads it at a fixed address)."""
+    t = _identities.get(device)
+    if t is None or t.numel() < n:
+        t = torch.arange(max(n, 2048), dtype=torch.int64, device=device)
+        _identities[device] = t
+    return t
+
+
 def moe_experts_grouped(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
                         limit: float) -> torch.Tensor:
     """The same function as moe_experts for steps with many tokens: assignments sorted by expert (stable), one [rows, width]
@@ -71,6 +83,18 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: 
     if n * top_k >= GROUPED_MIN_ROWS_PER_EXPERT * experts and not torch.cuda.is_current_stream_capturing():
         return moe_experts_grouped(h, idx, wts, gate_up, down, limit)
     code, stream = _hip.dtype_code3(h.dtype), _hip.stream()
+    if h.dtype != torch.float32 and _hip.load().swl_moe_expert_stationary_supported(n, width, ff, top_k, code):
+        # decode-sized 16-bit step: every expert's weights are read once, whatever the number of tokens that chose it
+        y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
+        _hip.call("swl_moe_expert_stationary", _hip.ptr(y), _hip.ptr(h), _hip.ptr(gate_up), _hip.ptr(idx), n, experts,
+                  width, ff, top_k, 1, float(limit), code, stream)
+        rows = torch.empty((n * top_k, width), dtype=h.dtype, device=h.device)
+        _hip.call("swl_moe_expert_stationary", _hip.ptr(rows), _hip.ptr(y), _hip.ptr(down), _hip.ptr(idx), n, experts,
+                  width, ff, top_k, 0, float(limit), code, stream)
+        out = torch.empty((n, width), dtype=h.dtype, device=h.device)
+        _hip.call("swl_moe_combine", _hip.ptr(out), _hip.ptr(rows), _hip.ptr(_identity(n * top_k, h.device)),
+                  _hip.ptr(wts), n, width, top_k, code, stream)
+        return out
     y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
     _hip.call("swl_moe_gate_up", _hip.ptr(y), _hip.ptr(h), _hip.ptr(gate_up), _hip.ptr(idx), n, width, ff, top_k,
               float(limit), code, stream)

@@ -125,6 +125,17 @@ def test_moe_router_and_experts(experts, top, n):
     down = torch.stack([W[f"e{e}.down"] for e in range(experts)]).cuda()
     got = moe_experts(h.cuda(), idx, wts, gate_up, down, limit)
     assert (got.cpu().double() - want).abs().max() < 2e-5
+    # 16-bit: decode-sized steps take the expert-stationary kernels (weights in registers, assignments grouped by expert in
+    # the kernel), large ones the sorted library products; same routing, results within 16-bit rounding of the oracle on
+    # the rounded inputs
+    hb = h.to(torch.bfloat16)
+    Wb = {k: v.to(torch.bfloat16).double() for k, v in W.items()}
+    Wb["router"], Wb["router.b"] = Wd["router"], Wd["router.b"]
+    want_b = O.moe_ff(hb.double(), Wb, "", mlp)
+    idx_b, wts_b = moe_route(hb.cuda(), W["router"].cuda(), W["router.b"].cuda(), top)
+    assert torch.equal(idx_b.cpu().long(), O.route(hb.double(), Wb, "", top)[0])
+    got_b = moe_experts(hb.cuda(), idx_b, wts_b, gate_up.to(torch.bfloat16), down.to(torch.bfloat16), limit)
+    assert (got_b.cpu().double() - want_b).abs().max() < 3e-2 * max(1.0, float(want_b.abs().max()))
 
 
 def _attention_case(heads, kv_heads, dim, vdim, window, n, softcap, seed, standout=None, dtype=torch.float32, tiled=False,
