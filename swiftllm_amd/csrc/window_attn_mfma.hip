@@ -74,14 +74,22 @@ __global__ __launch_bounds__(NW * 64, 1) void window_attn_mfma_kernel(
     constexpr int KS = D / 16;
     constexpr bool PIPE = HPW * D <= 512 && HPW * DV <= 512;
     vec4_t<T> qf[PIPE ? HPW : 1][KS], kf[PIPE ? HPW : 1][KS];
+    // element offsets inside a page: of each head's key / value slice (wave-uniform, divided once) and of this lane's fragment
+    int koff[HPW], voff[HPW];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        const int kv = __builtin_amdgcn_readfirstlane(min(h0 + hh, H - 1) / rep);
+        koff[hh] = kv * kWmTile * D;
+        voff[hh] = kv * DV * kWmTile;
+    }
+    const int lane_k = li * D + 4 * lq;             // A operand of S^T: key li, dims 4 lq ..
+    const int lane_v = li * kWmTile + 4 * lq;       // A operand of O^T: column li of a 16-column tile, keys 4 lq ..
     auto fetch_k = [&](int64_t blk) {
         const T *kblk = k_cache + blk * block_stride;
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
-            const int g = min(h0 + hh, H - 1);
-            const T *kr = kblk + (static_cast<int64_t>(g / rep) * kWmTile + li) * D + 4 * lq;    // A: key li, dims 4 lq ..
 #pragma unroll
-            for (int e = 0; e < KS; ++e) load4(kf[PIPE ? hh : 0][e], kr + e * 16);
+            for (int e = 0; e < KS; ++e) load4(kf[PIPE ? hh : 0][e], kblk + koff[hh] + lane_k + e * 16);
         }
     };
     if constexpr (PIPE) {
@@ -107,10 +115,8 @@ __global__ __launch_bounds__(NW * 64, 1) void window_attn_mfma_kernel(
         // a page's values transposed ([kv head][column][16 keys]), so this is one 8-byte load
         vec4_t<T> vfrag[PIPE ? HPW : 1][CT];
         auto fetch_v = [&](int hh) {
-            const int kv = min(h0 + hh, H - 1) / rep;
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct)
-                load4(vfrag[PIPE ? hh : 0][ct], vblk + (static_cast<int64_t>(kv) * DV + ct * 16 + li) * kWmTile + 4 * lq);
+            for (int ct = 0; ct < CT; ++ct) load4(vfrag[PIPE ? hh : 0][ct], vblk + voff[hh] + ct * 16 * kWmTile + lane_v);
         };
         if constexpr (PIPE) {
 #pragma unroll
@@ -126,7 +132,7 @@ __global__ __launch_bounds__(NW * 64, 1) void window_attn_mfma_kernel(
 #pragma unroll
                     for (int e = 0; e < KS; ++e) st = mfma16(kf[hh][e], qf[hh][e], st);
                 } else {
-                    const T *kr = kblk + (static_cast<int64_t>(g / rep) * kWmTile + li) * D + 4 * lq;
+                    const T *kr = kblk + koff[hh] + lane_k;
                     const T *qr = qrow + g * D + 4 * lq;
 #pragma unroll
                     for (int e = 0; e < KS; ++e) {

@@ -386,6 +386,39 @@ def test_other_sizes(tmp_path, dtype, tol):
         assert float((errs < tol).float().mean()) >= 0.7, errs
 
 
+def test_matrix_core_paths_in_the_model(tmp_path):
+    """Head sizes the matrix-core attention serves and expert widths the matrix-core expert products serve, in bfloat16:
+    whole prompt (tiles of 16 queries, experts through sorted library products), portions, and decoding (tiles of one query
+    with shared-out pages, expert-stationary products) against the oracle; and the per-token kernels on the same model."""
+    from swiftllm_amd.worker.kernels import window_attn
+    layers = [O.attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, window=40, mlp=O.moe_mlp(32, 4, 2)),
+              O.attention_layer(heads=2, kv_heads=1, dim=128, vdim=64, window=24, mlp=O.dense_mlp(128))]
+    cfg = O.make_config(width=128, vocab=96, layers=layers, loop=(0, 2, 2), max_positions=256)
+    W = O.random_weights(cfg, seed=21)
+    toks = tokens_for(cfg, 150, 4)
+    want = O.forward(cfg, W, toks)
+    model = make_model(tmp_path / "m", cfg, W, "bfloat16")
+    assert window_attn.tiles_supported(model.model_config.layers[0].mixer, torch.bfloat16)
+
+    def run(seq):
+        out = [model.step([entry(seq, toks[:100], 0)]), model.step([entry(seq, toks[100:131], 100)])]
+        out += [model.step([entry(seq, toks[i:i + 1], i)]) for i in range(131, 150)]
+        return torch.cat(out)
+
+    tiled = run(0)
+    saved = window_attn.TILES_MIN_TOKENS
+    window_attn.TILES_MIN_TOKENS = 1 << 30
+    try:
+        plain = run(1)
+    finally:
+        window_attn.TILES_MIN_TOKENS = saved
+    for got in (tiled, plain):
+        errs = torch.tensor([rel_err(got[i:i + 1], want[i:i + 1]) for i in range(got.shape[0])])
+        assert float((errs < BF16_TOL).float().mean()) >= 0.9, errs
+    errs = torch.tensor([rel_err(tiled[i:i + 1], plain[i:i + 1]) for i in range(tiled.shape[0])])
+    assert float((errs < BF16_TOL).float().mean()) >= 0.9, errs
+
+
 def test_no_loop_and_single_pass_loop(tmp_path):
     layers = [O.attention_layer(mlp=O.dense_mlp(32)), O.attention_layer(mlp=O.moe_mlp(16, 4, 2))]
     for name, loop in (("a", None), ("b", (1, 2, 1)), ("c", (0, 2, 3))):
