@@ -25,7 +25,7 @@ __device__ __forceinline__ float fast_tanh(float x) {
 }
 
 template <typename T, int D, int DV, int HPW, int NW>
-__global__ __launch_bounds__(NW * 64, 1) void window_attn_mfma_kernel(
+__global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk, int H, int G,
     int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
@@ -36,6 +36,7 @@ __global__ __launch_bounds__(NW * 64, 1) void window_attn_mfma_kernel(
     float *tk = s_all + nbuf * H * 256;
     constexpr int CT = DV / 16;         // 16-column tiles of the value head
     constexpr float kLog2e = 1.4426950408889634f;
+    constexpr float kLazy = 5.5f;
     const int tile = blockIdx.x;
     const int row0 = __builtin_amdgcn_readfirstlane(tile_row0[tile]), cnt = __builtin_amdgcn_readfirstlane(tile_cnt[tile]);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -190,7 +191,10 @@ __global__ __launch_bounds__(NW * 64, 1) void window_attn_mfma_kernel(
                 for (int r = 0; r < 4; ++r) cmax = fmaxf(cmax, ok[r] ? mixed[hh][r] : kNegBig);
                 cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
                 cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
-                const float mnew = fmaxf(mrun[hh], cmax);
+                // lazy running maximum: a row moves its reference only when a page raises it by more than kLazy, so the weights
+                // stay below e^kLazy instead of below 1 (fp32 sums; the hi + lo split keeps their relative precision at either
+                // scale) and alpha is exactly 1 on most pages: the accumulator rescale below is then skipped for the wave
+                const float mnew = cmax - mrun[hh] > kLazy ? cmax : mrun[hh];
                 const float alpha = fast_exp2((mrun[hh] - mnew) * kLog2e);
                 mrun[hh] = mnew;
                 vec4_t<T> phi, plo;
