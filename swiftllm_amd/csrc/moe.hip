@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_down_combine_kernel(T *out, c
 // per step however many tokens chose it (the per-assignment kernels above stream them once per token). GLU: n indexes ff,
 // the gate row n and the up row ff + n share the input fragments and meet in the clamped gated unit; X rows are tokens
 // (a / top). Otherwise (down projection) X rows are assignments and the output is the plain product, rounded to T.
-constexpr int kEsRows = 64;         // outputs per workgroup (16 per wave)
+constexpr int kEsRows = 64;         // outputs per workgroup at most (16 per wave; fewer waves when the grid would be small)
 constexpr int kEsTiles = 4;         // tiles of 16 assignments per pass over the weights
 constexpr int kEsMaxAssign = 1024;  // assignments per step (the sorted library path serves larger steps)
 
@@ -185,11 +185,11 @@ __global__ __launch_bounds__(kMoeThreads) void moe_expert_stationary_kernel(T *o
     const int li = lane & 15, lq = lane >> 4;
     if (threadIdx.x == 0) count = 0;
     __syncthreads();
-    for (int a = threadIdx.x; a < assignments; a += kMoeThreads)
+    for (int a = threadIdx.x; a < assignments; a += blockDim.x)
         if (expert_idx[a] == e) mine[atomicAdd(&count, 1)] = a;
     __syncthreads();
     const int m = count;
-    const int n0 = blockIdx.y * kEsRows + wave * 16;
+    const int n0 = (blockIdx.y * (blockDim.x >> 6) + wave) * 16;
     if (m == 0 || n0 >= N) return;
     const int nrow = min(n0 + li, N - 1);       // (rows past N compute a duplicate that is never stored)
     const T *wg = w + (static_cast<int64_t>(e) * (GLU ? 2 : 1) * N + nrow) * K + 4 * lq;
@@ -292,16 +292,19 @@ extern "C" int swl_moe_expert_stationary(void *out, const void *x, const void *w
     const int K = glu ? width : ff, N = glu ? ff : width;
     const int assignments = static_cast<int>(num_tokens * top);
     const size_t lds = 0;
-    const dim3 grid(static_cast<unsigned>(experts), static_cast<unsigned>((N + swl::kEsRows - 1) / swl::kEsRows));
+    // waves per workgroup: four, or fewer while the launch would have under ~1024 waves (a decode step must fill 256 CUs)
+    int nw = 4;
+    while (nw > 1 && static_cast<int64_t>(experts) * ((N + 16 * nw - 1) / (16 * nw)) * nw < 1024) nw >>= 1;
+    const dim3 grid(static_cast<unsigned>(experts), static_cast<unsigned>((N + 16 * nw - 1) / (16 * nw)));
     if (grid.y > 65535) return SWL_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     SWL_DISPATCH_DTYPE(dtype, T, {
         if (glu)
-            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, true>), grid, dim3(swl::kMoeThreads), lds, s,
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, true>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
                                assignments, K, N, top, limit);
         else
-            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, false>), grid, dim3(swl::kMoeThreads), lds, s,
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, false>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
                                assignments, K, N, top, limit);
     });
