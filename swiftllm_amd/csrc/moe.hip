@@ -175,13 +175,17 @@ constexpr int kEsTiles = 4;         // tiles of 16 assignments per pass over the
 constexpr int kEsMaxAssign = 1024;  // assignments per step (the sorted library path serves larger steps)
 
 template <typename T, bool GLU>
-__global__ __launch_bounds__(kMoeThreads) void moe_expert_stationary_kernel(T *out, const T *x, const T *w,
+__global__ __launch_bounds__(kMoeThreads, 2) void moe_expert_stationary_kernel(T *out, const T *x, const T *w,
                                                                             const int32_t *expert_idx, int assignments,
-                                                                            int K, int N, int top, float limit) {
+                                                                            int K, int N, int top, float limit, int ksplit) {
+    // ksplit = 1: every wave of the workgroup owns 16 outputs and the whole reduction. ksplit = waves of the workgroup: all
+    // waves own the SAME 16 outputs and a quarter (half) of the reduction each; their accumulators meet in LDS and wave 0
+    // finishes (short reductions and few outputs would otherwise leave most of the chip idle in a decode step).
     __shared__ int mine[kEsMaxAssign];
     __shared__ int count;
+    __shared__ float red[3][2 * kEsTiles][256];
     const int e = blockIdx.x;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
     const int li = lane & 15, lq = lane >> 4;
     if (threadIdx.x == 0) count = 0;
     __syncthreads();
@@ -189,11 +193,16 @@ __global__ __launch_bounds__(kMoeThreads) void moe_expert_stationary_kernel(T *o
         if (expert_idx[a] == e) mine[atomicAdd(&count, 1)] = a;
     __syncthreads();
     const int m = count;
-    const int n0 = (blockIdx.y * (blockDim.x >> 6) + wave) * 16;
-    if (m == 0 || n0 >= N) return;
+    const int n0 = ksplit > 1 ? blockIdx.y * 16 : (blockIdx.y * nwaves + wave) * 16;
+    if (m == 0 || (ksplit == 1 && n0 >= N)) return;
+    const int kper = K / ksplit;                       // (ksplit > 1: a multiple of 32, checked on the host)
+    const int kbeg = ksplit > 1 ? wave * kper : 0, kend = kbeg + kper;
     const int nrow = min(n0 + li, N - 1);       // (rows past N compute a duplicate that is never stored)
-    const T *wg = w + (static_cast<int64_t>(e) * (GLU ? 2 : 1) * N + nrow) * K + 4 * lq;
+    // this lane's share of a 32-wide reduction step: elements 8 lq .. 8 lq + 7 (one 16-byte load), fed to the matrix core as
+    // two 4-element halves — the same split on both operands, so the order inside a step does not matter
+    const T *wg = w + (static_cast<int64_t>(e) * (GLU ? 2 : 1) * N + nrow) * K + 8 * lq;
     const T *wu = wg + static_cast<int64_t>(N) * K;
+    const bool wide = (kper & 31) == 0 && ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) & 15) == 0 && (K & 7) == 0;
     for (int pass = 0; pass < m; pass += 16 * kEsTiles) {
         const int ntile = min(kEsTiles, (m - pass + 15) / 16);
         int arow[kEsTiles];
@@ -203,31 +212,82 @@ __global__ __launch_bounds__(kMoeThreads) void moe_expert_stationary_kernel(T *o
             const int i = pass + t * 16 + li;
             const int a = i < m ? mine[i] : -1;
             arow[t] = a;
-            xp[t] = x + static_cast<int64_t>(a < 0 ? 0 : (GLU ? a / top : a)) * K + 4 * lq;
+            xp[t] = x + static_cast<int64_t>(a < 0 ? 0 : (GLU ? a / top : a)) * K + 8 * lq;
         }
         float4_t accg[kEsTiles], accu[kEsTiles];
 #pragma unroll
         for (int t = 0; t < kEsTiles; ++t) accg[t] = accu[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-        for (int k0 = 0; k0 < K; k0 += 16) {
-            vec4_t<T> ag, au;
-            load4(ag, wg + k0);
-            if constexpr (GLU) load4(au, wu + k0);
+        if (wide) {
+#pragma unroll 2
+            for (int k0 = kbeg; k0 < kend; k0 += 32) {
+                const vec8_t<T> ag = load8(wg + k0);
+                vec8_t<T> au = vec8_t<T>{};
+                if constexpr (GLU) au = load8(wu + k0);
 #pragma unroll
-            for (int t = 0; t < kEsTiles; ++t) {
-                if (t < ntile) {
-                    vec4_t<T> b = vec4_t<T>{};
-                    if (arow[t] >= 0) load4(b, xp[t] + k0);
-                    accg[t] = mfma16(ag, b, accg[t]);
-                    if constexpr (GLU) accu[t] = mfma16(au, b, accu[t]);
+                for (int t = 0; t < kEsTiles; ++t) {
+                    if (t < ntile) {
+                        vec8_t<T> b = vec8_t<T>{};
+                        if (arow[t] >= 0) b = load8(xp[t] + k0);
+                        const vec4_t<T> b0 = {b[0], b[1], b[2], b[3]}, b1 = {b[4], b[5], b[6], b[7]};
+                        accg[t] = mfma16(vec4_t<T>{ag[0], ag[1], ag[2], ag[3]}, b0, accg[t]);
+                        accg[t] = mfma16(vec4_t<T>{ag[4], ag[5], ag[6], ag[7]}, b1, accg[t]);
+                        if constexpr (GLU) {
+                            accu[t] = mfma16(vec4_t<T>{au[0], au[1], au[2], au[3]}, b0, accu[t]);
+                            accu[t] = mfma16(vec4_t<T>{au[4], au[5], au[6], au[7]}, b1, accu[t]);
+                        }
+                    }
+                }
+            }
+        } else {
+            // 16-wide steps, 8-byte fragments (this lane: elements 4 lq .. 4 lq + 3 of the step)
+            const T *wg4 = wg - 4 * lq, *wu4 = wu - 4 * lq;
+#pragma unroll 4
+            for (int k0 = kbeg; k0 < kend; k0 += 16) {
+                vec4_t<T> ag, au;
+                load4(ag, wg4 + k0);
+                if constexpr (GLU) load4(au, wu4 + k0);
+#pragma unroll
+                for (int t = 0; t < kEsTiles; ++t) {
+                    if (t < ntile) {
+                        vec4_t<T> b = vec4_t<T>{};
+                        if (arow[t] >= 0) load4(b, xp[t] - 4 * lq + k0);
+                        accg[t] = mfma16(ag, b, accg[t]);
+                        if constexpr (GLU) accu[t] = mfma16(au, b, accu[t]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < kEsTiles; ++t) {
+            mfma_results_tie(accg[t]);
+            mfma_results_ready<4>(accu[t]);
+        }
+        if (ksplit > 1) {       // (workgroup-uniform) sum the waves' partial accumulators in wave 0
+            __syncthreads();    // (the previous pass's partials have been read)
+            if (wave > 0) {
+#pragma unroll
+                for (int t = 0; t < kEsTiles; ++t) {
+                    if (t < ntile) {
+                        *reinterpret_cast<float4_t *>(&red[wave - 1][2 * t][lane * 4]) = accg[t];
+                        if constexpr (GLU) *reinterpret_cast<float4_t *>(&red[wave - 1][2 * t + 1][lane * 4]) = accu[t];
+                    }
+                }
+            }
+            __syncthreads();
+            if (wave > 0) continue;
+            for (int o = 0; o + 1 < nwaves; ++o) {
+#pragma unroll
+                for (int t = 0; t < kEsTiles; ++t) {
+                    if (t < ntile) {
+                        accg[t] += *reinterpret_cast<const float4_t *>(&red[o][2 * t][lane * 4]);
+                        if constexpr (GLU) accu[t] += *reinterpret_cast<const float4_t *>(&red[o][2 * t + 1][lane * 4]);
+                    }
                 }
             }
         }
         // accumulator r of lane (li, lq): output row n0 + 4 lq + r of the assignment in column li
 #pragma unroll
         for (int t = 0; t < kEsTiles; ++t) {
-            mfma_results_tie(accg[t]);
-            mfma_results_ready<4>(accu[t]);
             if (t < ntile && arow[t] >= 0) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -292,21 +352,24 @@ extern "C" int swl_moe_expert_stationary(void *out, const void *x, const void *w
     const int K = glu ? width : ff, N = glu ? ff : width;
     const int assignments = static_cast<int>(num_tokens * top);
     const size_t lds = 0;
-    // waves per workgroup: four, or fewer while the launch would have under ~1024 waves (a decode step must fill 256 CUs)
-    int nw = 4;
-    while (nw > 1 && static_cast<int64_t>(experts) * ((N + 16 * nw - 1) / (16 * nw)) * nw < 1024) nw >>= 1;
-    const dim3 grid(static_cast<unsigned>(experts), static_cast<unsigned>((N + 16 * nw - 1) / (16 * nw)));
+    // Four waves per workgroup. With plenty of outputs each wave owns 16 of them; when that would launch under ~2048 waves
+    // (a decode step must fill 256 CUs x 4 SIMDs, with latency to hide) the four waves share 16 outputs and split the reduction.
+    const int nw = 4;
+    const int64_t tiles16 = (N + 15) / 16;
+    const int ksplit = (experts * tiles16 < 2048 && K % (32 * nw) == 0) ? nw : 1;
+    const dim3 grid(static_cast<unsigned>(experts),
+                    static_cast<unsigned>(ksplit > 1 ? tiles16 : (N + 16 * nw - 1) / (16 * nw)));
     if (grid.y > 65535) return SWL_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     SWL_DISPATCH_DTYPE(dtype, T, {
         if (glu)
             hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, true>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
-                               assignments, K, N, top, limit);
+                               assignments, K, N, top, limit, ksplit);
         else
             hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, false>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
-                               assignments, K, N, top, limit);
+                               assignments, K, N, top, limit, ksplit);
     });
     return swl::check_launch();
 }

@@ -18,12 +18,32 @@ __global__ __launch_bounds__(kPnThreads) void polynorm_kernel(T *out, const T *z
     const int64_t r = blockIdx.x;
     const T *zr = z + r * ff;
     float s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    for (int i = threadIdx.x; i < ff; i += kPnThreads) {
-        const float v = to_f(zr[i]);
-        const float v2 = v * v, v3 = v2 * v;
-        s1 += v2;
-        s2 += v2 * v2;
-        s3 += v3 * v3;
+    // 16-bit rows whose length is a multiple of 8 move 16 bytes per lane
+    bool wide = false;
+    if constexpr (sizeof(T) == 2) wide = (ff & 7) == 0 && ((reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    if constexpr (sizeof(T) == 2) {
+        if (wide) {
+            for (int i = threadIdx.x * 8; i < ff; i += kPnThreads * 8) {
+                const vec8_t<T> zv = load8(zr + i);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float v = to_f(zv[j]);
+                    const float v2 = v * v, v3 = v2 * v;
+                    s1 += v2;
+                    s2 += v2 * v2;
+                    s3 += v3 * v3;
+                }
+            }
+        }
+    }
+    if (!wide) {
+        for (int i = threadIdx.x; i < ff; i += kPnThreads) {
+            const float v = to_f(zr[i]);
+            const float v2 = v * v, v3 = v2 * v;
+            s1 += v2;
+            s2 += v2 * v2;
+            s3 += v3 * v3;
+        }
     }
     s1 = wave_allreduce_sum(s1);
     s2 = wave_allreduce_sum(s2);
@@ -45,6 +65,22 @@ __global__ __launch_bounds__(kPnThreads) void polynorm_kernel(T *out, const T *z
     const float n = static_cast<float>(ff);
     const float r1 = a / sqrtf(s1 / n + eps), r2 = b / sqrtf(s2 / n + eps), r3 = c / sqrtf(s3 / n + eps);
     T *orow = out + r * ff;
+    if constexpr (sizeof(T) == 2) {
+        if (wide) {
+            for (int i = threadIdx.x * 8; i < ff; i += kPnThreads * 8) {
+                const vec8_t<T> zv = load8(zr + i);
+                vec8_t<T> ov;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float v = to_f(zv[j]);
+                    const float v2 = v * v;
+                    ov[j] = to_t<T>(r1 * v + r2 * v2 + r3 * (v2 * v) + e);
+                }
+                store8(orow + i, ov);
+            }
+            return;
+        }
+    }
     for (int i = threadIdx.x; i < ff; i += kPnThreads) {
         const float v = to_f(zr[i]);
         const float v2 = v * v;

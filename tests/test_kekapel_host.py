@@ -13,11 +13,11 @@ import kekapel_oracle as O
 def test_layer_runs_follow_the_loop():
     from swiftllm_amd.model_config import KekapelModelConfig
     layers = [O.attention_layer(mlp=O.dense_mlp(32)) for _ in range(5)]
-    cfg = KekapelModelConfig(O.make_config(layers=layers, loop=(1, 3, 3)))
+    cfg = KekapelModelConfig(O.make_config(layers=layers, loop=(2, 4, 3)))
     assert [(r.layer, r.pass_index) for r in cfg.layer_runs] == [
-        (0, -1), (1, 0), (2, -1), (1, 1), (2, -1), (1, 2), (2, -1), (3, -1), (4, -1)]
+        (0, -1), (1, -1), (2, 0), (3, -1), (2, 1), (3, -1), (2, 2), (3, -1), (4, -1)]
     assert [r.index for r in cfg.layer_runs] == list(range(9))
-    assert [(i, t if first else -1) for i, t, first in O.layer_runs(O.make_config(layers=layers, loop=(1, 3, 3)))] == \
+    assert [(i, t if first else -1) for i, t, first in O.layer_runs(O.make_config(layers=layers, loop=(2, 4, 3)))] == \
         [(r.layer, r.pass_index) for r in cfg.layer_runs]
     # no loop, a loop of one pass (its step vector is still added), a loop over everything
     assert [r.pass_index for r in KekapelModelConfig(O.make_config(layers=layers)).layer_runs] == [-1] * 5
