@@ -22,7 +22,7 @@ PROMPTS = ["Life blooms like a flower, far away", "one two three four five",
 def main():
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--model-path", required=True)
-    ap.add_argument("--dtype", default="float16", choices=["float16", "bfloat16"])
+    ap.add_argument("--dtype", default="float16", choices=["float16", "bfloat16", "float32"])
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--use-dummy", action="store_true")
     args = ap.parse_args()
@@ -32,7 +32,7 @@ def main():
                                 max_blocks_per_seq=2048, max_batch_size=16, max_tokens_in_batch=2048 * 16,
                                 dtype=args.dtype, use_hip_graph=True)
     t0 = time.perf_counter()
-    model = swiftllm.LlamaModel(cfg)
+    model = swiftllm.build_model(cfg)      # the worker class the checkpoint's config.json names (LLaMA, Kekapel)
     model.load_weights()
     num_blocks = model.profile_num_blocks()
     model.init_kvcache_and_swap(min(num_blocks, 4096))

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     // Registers allowing (PIPE), the query fragments stay resident and the next page's key fragments are fetched while this
     // page's mix / softmax / value products run; the value fragments of a page are requested before its score products.
     constexpr int KS = D / 16;
-    constexpr bool PIPE = HPW * D <= 512 && HPW * DV <= 512;
+    constexpr bool PIPE = HPW * D <= 512 && HPW * DV <= 512 && (NW == 4 || HPW * (D + DV) <= 512);   // (eight waves: 256 registers each)
     vec4_t<T> qf[PIPE ? HPW : 1][KS], kf[PIPE ? HPW : 1][KS];
     // element offsets inside a page: of each head's key / value slice (wave-uniform, divided once) and of this lane's fragment
     int koff[HPW], voff[HPW];
