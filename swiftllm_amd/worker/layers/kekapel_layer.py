@@ -2,6 +2,8 @@
 bookkeeping around them (post-norm into the fp32 stream, the next input norm) is the model's fused step."""
 import torch
 
+from swiftllm_amd import _hip
+
 from ..kernels.linear import linear
 from ..kernels.moe import moe_experts, moe_route
 from ..kernels.polynorm import polynorm
@@ -13,7 +15,16 @@ def _project(a: torch.Tensor, w: torch.Tensor, skinny: bool) -> torch.Tensor:
     decode-sized batches, the BLAS otherwise); fp32: the BLAS in true fp32."""
     if a.dtype == torch.float32:
         return torch.nn.functional.linear(a, w)
-    return linear(a, w, skinny)
+    if skinny and not getattr(w, "_swl_blas_only", False):
+        try:
+            return linear(a, w, True)
+        except _hip.HipLibraryError as exc:
+            # a projection shape the hand-written decode GEMMs are not specialised for (they say so with the "not supported"
+            # code): this weight goes through the BLAS from here on; any other failure is a real one
+            if "code -2" not in str(exc):
+                raise
+            w._swl_blas_only = True
+    return linear(a, w, False)
 
 
 class KekapelAttention:

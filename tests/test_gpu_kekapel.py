@@ -213,7 +213,8 @@ def test_window_attention_against_dense_mask(heads, kv_heads, dim, vdim, window,
 
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,window,n", [
     (6, 2, 64, 64, 36, 150), (8, 2, 128, 128, 9, 70), (16, 4, 128, 64, 64, 131), (32, 8, 64, 64, 33, 90),
-    (5, 5, 64, 128, 200, 100), (1, 1, 64, 64, 16, 49), (3, 1, 128, 128, 1, 40), (32, 4, 128, 128, 17, 50)])
+    (5, 5, 64, 128, 200, 100), (1, 1, 64, 64, 16, 49), (3, 1, 128, 128, 1, 40), (32, 4, 128, 128, 17, 50),
+    (24, 8, 64, 64, 20, 60), (12, 4, 64, 64, 50, 90)])
 @pytest.mark.parametrize("dtype,atol", [(torch.float16, 4e-3), (torch.bfloat16, 3.2e-2)])
 def test_tiled_attention_matches_the_per_token_kernel(heads, kv_heads, dim, vdim, window, n, dtype, atol):
     """The matrix-core kernel (tiles of 16 queries, portions cut at odd places, a decoded token as a tile of one) against
