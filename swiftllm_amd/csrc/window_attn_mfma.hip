@@ -18,12 +18,6 @@ constexpr int kWmThreads = 256;
 constexpr int kWmWaves = 4;
 constexpr int kWmTile = 16;     // queries per tile = keys per page = MFMA edge
 
-__device__ __forceinline__ float fast_tanh(float x) {
-    // 1 - 2 / (e^{2x} + 1); exp2 overflow to inf gives exactly 1, underflow to 0 gives exactly -1
-    const float e = fast_exp2(x * 2.885390081777927f);
-    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
-}
-
 template <typename T, int D, int DV, int HPW, int NW>
 __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
@@ -36,13 +30,13 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     float *tk = s_all + nbuf * H * 256;
     constexpr int CT = DV / 16;         // 16-column tiles of the value head
     constexpr float kLog2e = 1.4426950408889634f;
-    constexpr float kLazy = 5.5f;
+    constexpr float kLazy = 8.0f;       // (base-2 units: weights stay below 2^8)
     const int tile = blockIdx.x;
     const int row0 = __builtin_amdgcn_readfirstlane(tile_row0[tile]), cnt = __builtin_amdgcn_readfirstlane(tile_cnt[tile]);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // (tells the compiler that it is wave-uniform)
     const int li = lane & 15, lq = lane >> 4;       // query (or operand row) index; quarter
-    for (int i = tid; i < H * H; i += NW * 64) tk[i] = talk[i];
+    for (int i = tid; i < H * H; i += NW * 64) tk[i] = talk[i] * kLog2e;     // mixed scores come out in base-2 exponent units
     __syncthreads();
     const int p0 = __builtin_amdgcn_readfirstlane(tok_pos[row0]);
     const int32_t *bt = block_table + static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tok_seq[row0])) * max_blocks_per_seq;
@@ -57,7 +51,8 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
         kb0 += per * static_cast<int>(blockIdx.y);
         kb1 = min(kb1, kb0 + per - 1);
     }
-    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+    // cap * tanh(s * scale / cap) = cap - 2 cap / (2^(s * c1) + 1) with c1 = 2 log2(e) scale / cap: five operations per score
+    const float c1 = softcap > 0.f ? 2.0f * kLog2e * scale / softcap : 0.f, cap2 = -2.0f * softcap;
 
     float4_t acc[HPW][CT];
     float mrun[HPW], lrun[HPW];
@@ -147,9 +142,10 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
                 // st[r] = S^T[key 4 lq + r][query li]
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float v = st[r] * scale;
-                    if (softcap > 0.f) v = softcap * fast_tanh(v * inv_cap);
-                    st[r] = v;
+                    if (softcap > 0.f)      // (2^x overflowing to inf gives exactly cap, underflowing to 0 exactly -cap)
+                        st[r] = fmaf(cap2, __builtin_amdgcn_rcpf(fast_exp2(st[r] * c1) + 1.0f), softcap);
+                    else
+                        st[r] *= scale;
                 }
                 *reinterpret_cast<float4_t *>(&s_lds[(g * 64 + lane) * 4]) = st;
             }
@@ -195,13 +191,13 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
                 // stay below e^kLazy instead of below 1 (fp32 sums; the hi + lo split keeps their relative precision at either
                 // scale) and alpha is exactly 1 on most pages: the accumulator rescale below is then skipped for the wave
                 const float mnew = cmax - mrun[hh] > kLazy ? cmax : mrun[hh];
-                const float alpha = fast_exp2((mrun[hh] - mnew) * kLog2e);
+                const float alpha = fast_exp2(mrun[hh] - mnew);
                 mrun[hh] = mnew;
                 vec4_t<T> phi, plo;
                 float psum = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float pv = ok[r] ? fast_exp2((mixed[hh][r] - mnew) * kLog2e) : 0.f;
+                    const float pv = ok[r] ? fast_exp2(mixed[hh][r] - mnew) : 0.f;
                     psum += pv;
                     phi[r] = to_t<T>(pv);
                     plo[r] = to_t<T>(pv - to_f(phi[r]));
@@ -268,15 +264,15 @@ template <typename T>
 __global__ __launch_bounds__(256) void window_attn_combine_kernel(T *out, const float *part_o, const float *part_ml,
                                                                   int64_t rows, int dv, int nsplit) {
     const int64_t row = blockIdx.x;     // (token, head)
-    float mx = kNegBig;
+    float mx = kNegBig;     // (the maxima are in base-2 exponent units)
     for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_ml[(s * rows + row) * 2]);
     float den = 0.f;
     for (int s = 0; s < nsplit; ++s)
-        den += expf(part_ml[(s * rows + row) * 2] - mx) * part_ml[(s * rows + row) * 2 + 1];
+        den += exp2f(part_ml[(s * rows + row) * 2] - mx) * part_ml[(s * rows + row) * 2 + 1];
     for (int c = threadIdx.x; c < dv; c += blockDim.x) {
         float a = 0.f;
         for (int s = 0; s < nsplit; ++s)
-            a += expf(part_ml[(s * rows + row) * 2] - mx) * part_o[(s * rows + row) * dv + c];
+            a += exp2f(part_ml[(s * rows + row) * 2] - mx) * part_o[(s * rows + row) * dv + c];
         out[row * dv + c] = to_t<T>(a / den);
     }
 }
