@@ -5,7 +5,8 @@
 // over the waves: wave w owns heads [w * HPW, (w + 1) * HPW) for the score products AND for the outputs, and the capped
 // scores of all heads meet in LDS in between. Per 16-key page:
 //   1. S^T_g = K_kv(g) Q_g^T      (16 keys x 16 queries, MFMA 16x16x16, fp32 accumulate), scale, tanh cap -> LDS [H][256] fp32
-//   2. mixed_h = sum_g talk[h][g] S^T_g   (fp32 VALU, talk from scalar loads), window mask, online softmax per (h, query)
+//   2. mixed_h = sum_g talk[h][g] S^T_g   (fp32 VALU, talk as LDS broadcasts), window mask, online softmax per (h, query)
+//      with a lazy running maximum, everything in base-2 exponent units
 //   3. O^T_h += V^T_kv(h) P^T_h   with the fp32 weights split into two 16-bit terms (hi + lo): the product keeps ~16 bits of
 //      every weight although the matrix core takes 16-bit operands.
 // The transposed products keep the query index on the lanes' low four bits in every stage, so the softmax statistics of a

@@ -18,10 +18,17 @@ from .block_mgmt import (
     gather_allocated_blocks_and_unset,
 )
 from .block_swapping import swap_blocks
+# operators of models beyond the reference's LLaMA (fp32 residual stream, windowed head-mixed attention, PolyNorm, MoE)
+from .layernorm import add_layernorm, embed_positions, layernorm
+from .window_attn import qknorm_and_store_kv, window_attention
+from .polynorm import polynorm
+from .moe import moe_experts, moe_route
 
 __all__ = [
     "linear", "rmsnorm_inplace", "fused_add_rmsnorm_inplace", "rotary_embedding_inplace",
     "store_kvcache", "prefill_attention", "paged_attention", "silu_and_mul_inplace",
     "set_block_table_and_num_seq_alloc_blocks", "unset_block_table_and_num_seq_alloc_blocks",
     "gather_allocated_blocks_and_unset", "swap_blocks",
+    "add_layernorm", "embed_positions", "layernorm", "qknorm_and_store_kv", "window_attention", "polynorm", "moe_experts",
+    "moe_route",
 ]

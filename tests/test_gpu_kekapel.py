@@ -3,7 +3,6 @@ token-by-token decoding, portions, unequal batches, reused blocks and rows, wind
 through the Engine and its scheduler. Configurations and weights are made here (small, random, seeded)."""
 import asyncio
 import json
-import math
 import os
 
 import pytest
