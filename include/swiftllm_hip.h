@@ -521,8 +521,10 @@ int swl_qknorm_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_c
  * out[T, H * vdim]; token t attends keys [max(0, p - window + 1), p] of its sequence (window 0: all), p = tok_pos[t];
  * score = softcap * tanh(q.k * scale / softcap) (softcap 0: none), mixed over heads by talk[H, H] (fp32), softmax, values.
  * H <= 32, H * vdim <= 8192. dtype may be SWL_F32. */
+/* talk may be NULL (no head mixing). rel (may be NULL): fp32 [num_q_heads, rel_len], a bias added to the (mixed) score of
+ * head h at distance query position - key position (distances beyond rel_len - 1 take the last entry). */
 int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
-                    const int32_t *tok_seq, const int32_t *tok_pos, const float *talk, int64_t num_tokens,
+                    const int32_t *tok_seq, const int32_t *tok_pos, const float *talk, const float *rel, int32_t rel_len, int64_t num_tokens,
                     int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride,
                     int32_t window, float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride,
                     int32_t dtype, swl_stream_t stream);
@@ -536,7 +538,7 @@ int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v
 int swl_window_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int32_t dtype);
 int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
                           const int32_t *tok_seq, const int32_t *tok_pos, const int32_t *tile_row0,
-                          const int32_t *tile_cnt, const float *talk, int32_t num_tiles, int32_t num_q_heads,
+                          const int32_t *tile_cnt, const float *talk, const float *rel, int32_t rel_len, int32_t num_tiles, int32_t num_q_heads,
                           int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window,
                           float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride,
                           int32_t key_splits, float *scratch, int64_t num_tokens, int32_t dtype, swl_stream_t stream);
@@ -570,6 +572,58 @@ int swl_moe_combine(void *out, const void *rows, const int64_t *where, const flo
                     int32_t width, int32_t top, int32_t dtype, swl_stream_t stream);
 int swl_moe_down_combine(void *out, const void *y, const void *down, const int32_t *expert_idx, const float *expert_w,
                          int64_t num_tokens, int32_t width, int32_t ff, int32_t top, int32_t dtype, swl_stream_t stream);
+
+/* Squared-ReLU experts and routers that weigh by the softmax over ALL experts. swl_moe_route_scores: the `top` experts with
+ * the largest fp32 logits router h (+ bias, may be NULL); weights = scale * softmax(all logits)[chosen], not renormalised.
+ * swl_moe_up_relu2: y[T * top, ff] = relu(up[e] h)^2, up [experts, ff, width]. swl_moe_expert_stationary with glu = 2 is its
+ * matrix-core form. swl_relu_sq: y[r][f] = relu(z[r * in_stride + f])^2. dtype may be SWL_F32. */
+int swl_moe_route_scores(int32_t *idx_out, float *w_out, const void *h, const float *router, const float *bias,
+                         int64_t num_tokens, int32_t width, int32_t experts, int32_t top, float scale, int32_t dtype,
+                         swl_stream_t stream);
+int swl_moe_up_relu2(void *y, const void *h, const void *up, const int32_t *expert_idx, int64_t num_tokens, int32_t width,
+                     int32_t ff, int32_t top, int32_t dtype, swl_stream_t stream);
+int swl_relu_sq(void *y, const void *z, int64_t num_rows, int32_t ff, int64_t in_stride, int32_t dtype, swl_stream_t stream);
+
+/* ---- q/k RMS norm over the whole projection + KV store (pool layout of swl_qknorm_store_kv) -------------------------------
+ * q <- q / rms(q over all heads) * q_w[heads * dim] * (1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)); keys likewise
+ * (no multiplier) into the pool, values copied. k_cache NULL: the row holds queries only. dtype may be SWL_F32. */
+int swl_qknorm_full_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_cache, void *v_cache,
+                             const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                             int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim,
+                             int64_t tok_stride, int32_t max_blocks_per_seq, int64_t block_stride, float eps,
+                             float temp_coef, int32_t temp_every, int32_t dtype, swl_stream_t stream);
+
+/* ---- fp32 stream with RMS norms, gated sublayer results and causal input convolutions (csrc/rms_stream.hip) --------------
+ * swl_gated_add_rmsnorm: y = m (+ sigmoid(m2_gate[t]) * m2); y *= sigmoid(r + r_bias); x += y / rms(y) * w1; out = x / rms(x)
+ * * w2. m NULL: only the output norm, of rows row_idx when given. Per-sequence state: `state` is the base of the state slots
+ * (fp32, slot_stride floats apart); tok_state[t] = slot * 2 + parity, tok_start[t] = position of the first token of t's
+ * portion. swl_causal_conv_state: out = (h if add_input) + causal convolution of h over time with w [channels, taps] (fp32),
+ * the carried inputs at tail_off inside the slot ([2][taps - 1][channels] floats). dtype may be SWL_F32. */
+int swl_gated_add_rmsnorm(float *x, const void *m, const void *m2, const void *m2_gate, int64_t m2_gate_stride,
+                          const void *r, int64_t r_stride, const float *r_bias, const float *w1, void *out, const float *w2,
+                          const int32_t *row_idx, float eps, int64_t num_rows, int32_t width, int32_t dtype,
+                          swl_stream_t stream);
+int swl_causal_conv_state(void *out, int64_t out_stride, const void *h, int64_t h_stride, const float *w, float *state,
+                          int64_t slot_stride, int64_t tail_off, const int32_t *tok_pos, const int32_t *tok_start,
+                          const int32_t *tok_state, const int32_t *tok_seq, int64_t num_tokens, int32_t channels,
+                          int32_t taps, int32_t add_input, int32_t dtype, swl_stream_t stream);
+
+/* ---- gated delta rule (csrc/delta_rule.hip) --------------------------------------------------------------------------------
+ * swl_delta_prep: proj rows [q | k | v | gate | b | a] -> qn, kn [T, qk heads * dim], vv [T, heads * vdim], beta, decay
+ * [T, heads], all fp32 (convolution + SiLU, unit norms, sigmoid, exp(-exp(A_log) softplus(a + dt_bias))).
+ * swl_delta_rule: o[T, heads * vdim] (fp32) and the states [heads, dim, vdim] at s_off inside the slots, one portion per
+ * (seq_row0, seq_cnt) entry. swl_gated_head_rmsnorm: out = o / rms(o over vdim) * w[vdim] * silu(gate). */
+int swl_delta_prep(float *qn, float *kn, float *vv, float *beta, float *decay, const void *proj, int64_t proj_stride,
+                   const float *conv_w, const float *a_log, const float *dt_bias, float *state, int64_t slot_stride,
+                   int64_t tail_off, const int32_t *tok_pos, const int32_t *tok_start, const int32_t *tok_state,
+                   const int32_t *tok_seq, int64_t num_tokens, int32_t num_heads, int32_t num_qk_heads, int32_t dim,
+                   int32_t vdim, int32_t taps, int32_t dtype, swl_stream_t stream);
+int swl_delta_rule(float *o, const float *qn, const float *kn, const float *vv, const float *beta, const float *decay,
+                   float *state, int64_t slot_stride, int64_t s_off, const int32_t *seq_row0, const int32_t *seq_cnt,
+                   const int32_t *tok_pos, const int32_t *tok_state, int32_t num_seqs, int32_t num_heads,
+                   int32_t num_qk_heads, int32_t dim, int32_t vdim, swl_stream_t stream);
+int swl_gated_head_rmsnorm(void *out, const float *o, const void *gate, int64_t gate_stride, const float *w, float eps,
+                           int64_t num_tokens, int32_t num_heads, int32_t vdim, int32_t dtype, swl_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -98,9 +98,9 @@ SIGNATURES = {
     "swl_add_layernorm": [_P, _P, _F32, _P, _P, _P, _P, _P, _P, _P, _F32, _I64, _I32, _I32, _P],
     "swl_qknorm_store_kv": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _I64, _F32, _I32,
                             _P],
-    "swl_window_attn": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32, _I32,
+    "swl_window_attn": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32, _I32,
                         _I64, _I32, _P],
-    "swl_window_attn_tiles": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32,
+    "swl_window_attn_tiles": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32,
                               _I32, _I64, _I32, _P, _I64, _I32, _P],
     "swl_polynorm": [_P, _P, _F32, _F32, _F32, _F32, _F32, _I64, _I32, _I32, _P],
     "swl_moe_route": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
@@ -109,6 +109,17 @@ SIGNATURES = {
     "swl_glu_clamp": [_P, _P, _I64, _I32, _F32, _I32, _P],
     "swl_moe_combine": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _P],
     "swl_moe_down_combine": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
+    "swl_moe_route_scores": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _P],
+    "swl_moe_up_relu2": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
+    "swl_relu_sq": [_P, _P, _I64, _I32, _I64, _I32, _P],
+    "swl_qknorm_full_store_kv": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _I64, _F32,
+                                 _F32, _I32, _I32, _P],
+    "swl_gated_add_rmsnorm": [_P, _P, _P, _P, _I64, _P, _I64, _P, _P, _P, _P, _P, _F32, _I64, _I32, _I32, _P],
+    "swl_causal_conv_state": [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
+    "swl_delta_prep": [_P, _P, _P, _P, _P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32,
+                       _I32, _I32, _I32, _P],
+    "swl_delta_rule": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
+    "swl_gated_head_rmsnorm": [_P, _P, _P, _I64, _P, _F32, _I64, _I32, _I32, _I32, _P],
 }
 # Entry points that do not follow the "int rc = f(...)" convention.
 _SPECIAL = {

@@ -35,6 +35,8 @@ SOURCES = [
     "window_attn_mfma.hip",
     "polynorm.hip",
     "moe.hip",
+    "rms_stream.hip",
+    "delta_rule.hip",
 ]
 # What a model family's worker calls (the shared pieces included): `build(only=MODEL_SOURCES[...])` compiles just these, so
 # that the first use from a fresh checkout does not pay for kernels the model never launches. A later full build compiles
@@ -44,8 +46,10 @@ MODEL_SOURCES = {
     "llama": list(SOURCES[:14]),
     "Kekapel": _SHARED + ["layernorm.hip", "qknorm_kv.hip", "window_attn.hip", "window_attn_mfma.hip",
                           "polynorm.hip", "moe.hip"],
+    "Lorulix": _SHARED + ["layernorm.hip", "qknorm_kv.hip", "window_attn.hip", "window_attn_mfma.hip", "moe.hip",
+                          "rms_stream.hip", "delta_rule.hip"],
 }
-HEADERS = ["swl_common.h", "attend_block.h", os.path.join(ROOT, "include", "swiftllm_hip.h")]
+HEADERS = ["swl_common.h", "attend_block.h", "conv_tail.h", os.path.join(ROOT, "include", "swiftllm_hip.h")]
 LIB = os.path.join(HERE, "libswiftllm_hip.so")
 OBJ_DIR = os.path.join(HERE, "build")
 ARCH = "gfx950"

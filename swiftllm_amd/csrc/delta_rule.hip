@@ -1,0 +1,260 @@
+// delta_rule.hip — the gated delta rule as a recurrent mixer, for any mixture of prompt portions and decoded tokens.
+//
+// Per head a state S [dim, vdim] (fp32, in the sequence's state slot) is carried from token to token:
+//     S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+// with unit vectors q (scaled by dim^-1/2) and k, beta in (0, 1) and a decay g in (0, 1).
+//
+//   swl_delta_prep:  one workgroup per token. The fused input projection row [q | k | v | gate | b | a] -> short causal
+//                    convolution + SiLU on q, k, v (carried inputs: conv_tail.h), unit norms of the q / k heads,
+//                    beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias)); everything after the loads is fp32.
+//   swl_delta_rule:  one workgroup per (portion, head). The columns of S are independent recurrences, so a column belongs
+//                    to L adjacent lanes, each holding dim / L of its elements in registers; per token the lanes exchange
+//                    three partial dot products (S^T k, S^T q, k . q) through DPP and o = S^T q + u (k . q) needs no second
+//                    pass over the state. q, k, v, beta, g of 16 tokens at a time are staged in LDS. The token loop is
+//                    sequential whatever the cut of the sequence into steps: the same operations in the same order.
+//   swl_gated_head_rmsnorm: out = o / rms(o over vdim) * w * silu(gate), per head.
+#include "swl_common.h"
+#include "conv_tail.h"
+
+namespace swl {
+
+constexpr int kDpThreads = 256;
+constexpr int kDrChunk = 16;        // tokens staged per round
+
+__device__ __forceinline__ float dr_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+template <typename T>
+__global__ __launch_bounds__(kDpThreads) void delta_prep_kernel(
+    float *qn, float *kn, float *vv, float *beta, float *decay, const T *proj, int64_t proj_stride, const float *conv_w,
+    const float *a_log, const float *dt_bias, float *state, int64_t slot_stride, int64_t tail_off, const int32_t *tok_pos,
+    const int32_t *tok_start, const int32_t *tok_state, const int32_t *tok_seq, int64_t num_tokens, int H, int G, int d,
+    int dv, int taps) {
+    extern __shared__ float act[];      // [2 G d + H dv] convolved, activated channels
+    const int64_t t = blockIdx.x;
+    const int qk = G * d, C = 2 * qk + H * dv;
+    const T *row = proj + t * proj_stride;
+    const ConvTail tail(state, slot_stride, tail_off, tok_pos, tok_start, tok_state, tok_seq, num_tokens, C, taps, t);
+    for (int c = threadIdx.x; c < C; c += kDpThreads) {
+        const float cur = to_f(row[c]);
+        const float a = tail.conv(proj, proj_stride, conv_w, c, cur);
+        act[c] = a * dr_sigmoid(a);
+        tail.save(proj, proj_stride, c, cur);
+    }
+    __syncthreads();
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const float qscale = 1.0f / sqrtf(static_cast<float>(d));
+    for (int hh = wave; hh < 2 * G; hh += kDpThreads / 64) {
+        const float *src = act + hh * d;
+        float ss = 0.f;
+        for (int e = lane; e < d; e += 64) ss += src[e] * src[e];
+        ss = wave_allreduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss + 1e-6f);
+        if (hh < G) {
+            float *dst = qn + t * qk + hh * d;
+            for (int e = lane; e < d; e += 64) dst[e] = src[e] * r * qscale;
+        } else {
+            float *dst = kn + t * qk + (hh - G) * d;
+            for (int e = lane; e < d; e += 64) dst[e] = src[e] * r;
+        }
+    }
+    for (int i = threadIdx.x; i < H * dv; i += kDpThreads) vv[t * H * dv + i] = act[2 * qk + i];
+    for (int h = threadIdx.x; h < H; h += kDpThreads) {
+        const float b = to_f(row[C + H * dv + h]), a = to_f(row[C + H * dv + H + h]);
+        beta[t * H + h] = dr_sigmoid(b);
+        const float z = a + dt_bias[h];
+        const float sp = z > 20.f ? z : log1pf(expf(z));
+        decay[t * H + h] = expf(-expf(a_log[h]) * sp);
+    }
+}
+
+template <int L>
+__device__ __forceinline__ float dr_group_sum(float v) {
+    return group_allreduce_sum<L>(v);
+}
+
+template <int MAXDS, int L>
+__global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float *qn, const float *kn, const float *vv,
+                                                          const float *beta, const float *decay, float *state,
+                                                          int64_t slot_stride, int64_t s_off, const int32_t *seq_row0,
+                                                          const int32_t *seq_cnt, const int32_t *tok_pos,
+                                                          const int32_t *tok_state, int H, int G, int d, int dv) {
+    extern __shared__ float lds[];
+    float *qs = lds;                        // [chunk][d]
+    float *ks = qs + kDrChunk * d;          // [chunk][d]
+    float *vs = ks + kDrChunk * d;          // [chunk][dv]
+    float *bs = vs + kDrChunk * dv;         // [chunk]
+    float *gs = bs + kDrChunk;              // [chunk]
+    const int seq = blockIdx.x, h = blockIdx.y;
+    const int row0 = seq_row0[seq], cnt = seq_cnt[seq];
+    const int kvh = h / (H / G);
+    const int col = threadIdx.x / L, l = threadIdx.x % L;
+    const int ds = d / L, i0 = l * ds;
+    float *S = state + static_cast<int64_t>(tok_state[row0] >> 1) * slot_stride + s_off + static_cast<int64_t>(h) * d * dv;
+    float s[MAXDS];
+    const bool fresh = tok_pos[row0] == 0;      // a sequence starts from the zero state whatever the slot held
+#pragma unroll
+    for (int i = 0; i < MAXDS; ++i) s[i] = (i < ds && !fresh) ? S[static_cast<int64_t>(i0 + i) * dv + col] : 0.f;
+    const int qk = G * d, hv = H * dv;
+    for (int c0 = 0; c0 < cnt; c0 += kDrChunk) {
+        const int cn = min(kDrChunk, cnt - c0);
+        __syncthreads();        // the previous chunk has been consumed
+        for (int i = threadIdx.x; i < cn * d; i += blockDim.x) {
+            const int j = i / d, e = i - j * d;
+            const int64_t r = row0 + c0 + j;
+            qs[i] = qn[r * qk + kvh * d + e];
+            ks[i] = kn[r * qk + kvh * d + e];
+        }
+        for (int i = threadIdx.x; i < cn * dv; i += blockDim.x) {
+            const int j = i / dv, e = i - j * dv;
+            vs[i] = vv[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + e];
+        }
+        for (int j = threadIdx.x; j < cn; j += blockDim.x) {
+            bs[j] = beta[static_cast<int64_t>(row0 + c0 + j) * H + h];
+            gs[j] = decay[static_cast<int64_t>(row0 + c0 + j) * H + h];
+        }
+        __syncthreads();
+        for (int j = 0; j < cn; ++j) {
+            const float g = gs[j], b = bs[j];
+            const float *kj = ks + j * d + i0, *qj = qs + j * d + i0;
+            float sk = 0.f, sq = 0.f, kq = 0.f;
+#pragma unroll
+            for (int i = 0; i < MAXDS; ++i) {
+                if (i < ds) {
+                    s[i] *= g;
+                    sk += s[i] * kj[i];
+                    sq += s[i] * qj[i];
+                    kq += kj[i] * qj[i];
+                }
+            }
+            sk = dr_group_sum<L>(sk);
+            sq = dr_group_sum<L>(sq);
+            kq = dr_group_sum<L>(kq);
+            const float u = b * (vs[j * dv + col] - sk);
+#pragma unroll
+            for (int i = 0; i < MAXDS; ++i)
+                if (i < ds) s[i] += kj[i] * u;
+            if (l == 0) o[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + col] = sq + u * kq;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MAXDS; ++i)
+        if (i < ds) S[static_cast<int64_t>(i0 + i) * dv + col] = s[i];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_head_rmsnorm_kernel(T *out, const float *o, const T *gate, int64_t gate_stride,
+                                                                 const float *w, float eps, int H, int dv) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int h = wave; h < H; h += 4) {
+        const float *src = o + (t * H + h) * dv;
+        float ss = 0.f;
+        for (int e = lane; e < dv; e += 64) ss += src[e] * src[e];
+        ss = wave_allreduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss / static_cast<float>(dv) + eps);
+        for (int e = lane; e < dv; e += 64) {
+            const float z = to_f(gate[t * gate_stride + h * dv + e]);
+            out[(t * H + h) * dv + e] = to_t<T>(src[e] * r * w[e] * (z * dr_sigmoid(z)));
+        }
+    }
+}
+
+// lanes per state column: as many as keep at least 8 elements per lane, a power of two that divides dim, at most 16 and at
+// most 1024 threads per workgroup
+inline int dr_lanes(int d, int dv) {
+    int L = 16;
+    while (L > 1 && (d % L || d / L < 8 || static_cast<int64_t>(dv) * L > 1024)) L >>= 1;
+    return L;
+}
+
+template <int L>
+int launch_dr(int ds, dim3 grid, dim3 block, size_t lds, hipStream_t s, float *o, const float *qn, const float *kn,
+              const float *vv, const float *beta, const float *decay, float *state, int64_t slot_stride, int64_t s_off,
+              const int32_t *seq_row0, const int32_t *seq_cnt, const int32_t *tok_pos, const int32_t *tok_state, int H,
+              int G, int d, int dv) {
+#define SWL_DR_LAUNCH(M)                                                                                                     \
+    hipLaunchKernelGGL((delta_rule_kernel<M, L>), grid, block, lds, s, o, qn, kn, vv, beta, decay, state, slot_stride, s_off, \
+                       seq_row0, seq_cnt, tok_pos, tok_state, H, G, d, dv)
+    if (ds <= 8) SWL_DR_LAUNCH(8);
+    else if (ds <= 16) SWL_DR_LAUNCH(16);
+    else if (ds <= 32) SWL_DR_LAUNCH(32);
+    else if (ds <= 64) SWL_DR_LAUNCH(64);
+    else if (ds <= 128) SWL_DR_LAUNCH(128);
+    else return SWL_ERR_UNSUPPORTED;
+#undef SWL_DR_LAUNCH
+    return check_launch();
+}
+
+} // namespace swl
+
+extern "C" int swl_delta_prep(float *qn, float *kn, float *vv, float *beta, float *decay, const void *proj,
+                              int64_t proj_stride, const float *conv_w, const float *a_log, const float *dt_bias,
+                              float *state, int64_t slot_stride, int64_t tail_off, const int32_t *tok_pos,
+                              const int32_t *tok_start, const int32_t *tok_state, const int32_t *tok_seq,
+                              int64_t num_tokens, int32_t num_heads, int32_t num_qk_heads, int32_t dim, int32_t vdim,
+                              int32_t taps, int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || num_heads <= 0 || num_qk_heads <= 0 || dim <= 0 || vdim <= 0 || taps < 1) return SWL_ERR_BAD_ARG;
+    if (num_heads % num_qk_heads) return SWL_ERR_BAD_ARG;
+    const int64_t C = 2LL * num_qk_heads * dim + static_cast<int64_t>(num_heads) * vdim;
+    if (proj_stride < C + static_cast<int64_t>(num_heads) * vdim + 2 * num_heads) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!qn || !kn || !vv || !beta || !decay || !proj || !conv_w || !a_log || !dt_bias || !tok_pos || !tok_start || !tok_seq)
+        return SWL_ERR_BAD_ARG;
+    if (taps > 1 && (!state || !tok_state)) return SWL_ERR_BAD_ARG;
+    const size_t lds = static_cast<size_t>(C) * sizeof(float);
+    if (num_tokens > 0x7fffffffLL || lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::delta_prep_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kDpThreads), lds,
+                           static_cast<hipStream_t>(stream), qn, kn, vv, beta, decay, static_cast<const T *>(proj),
+                           proj_stride, conv_w, a_log, dt_bias, state, slot_stride, tail_off, tok_pos, tok_start,
+                           tok_state, tok_seq, num_tokens, num_heads, num_qk_heads, dim, vdim, taps);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_delta_rule(float *o, const float *qn, const float *kn, const float *vv, const float *beta,
+                              const float *decay, float *state, int64_t slot_stride, int64_t s_off,
+                              const int32_t *seq_row0, const int32_t *seq_cnt, const int32_t *tok_pos,
+                              const int32_t *tok_state, int32_t num_seqs, int32_t num_heads, int32_t num_qk_heads,
+                              int32_t dim, int32_t vdim, swl_stream_t stream) {
+    if (num_seqs < 0 || num_heads <= 0 || num_qk_heads <= 0 || dim <= 0 || vdim <= 0 || num_heads % num_qk_heads)
+        return SWL_ERR_BAD_ARG;
+    if (num_seqs == 0) return SWL_OK;
+    if (!o || !qn || !kn || !vv || !beta || !decay || !state || !seq_row0 || !seq_cnt || !tok_pos || !tok_state)
+        return SWL_ERR_BAD_ARG;
+    if (vdim > 1024 || num_heads > 65535) return SWL_ERR_UNSUPPORTED;
+    const int L = swl::dr_lanes(dim, vdim);
+    const int ds = dim / L;
+    const size_t lds = (static_cast<size_t>(swl::kDrChunk) * (2 * dim + vdim + 2)) * sizeof(float);
+    if (lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads)), block(static_cast<unsigned>(vdim * L));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define SWL_DR_L(LL)                                                                                                         \
+    case LL: return swl::launch_dr<LL>(ds, grid, block, lds, s, o, qn, kn, vv, beta, decay, state, slot_stride, s_off,       \
+                                       seq_row0, seq_cnt, tok_pos, tok_state, num_heads, num_qk_heads, dim, vdim)
+    switch (L) {
+        SWL_DR_L(1);
+        SWL_DR_L(2);
+        SWL_DR_L(4);
+        SWL_DR_L(8);
+        SWL_DR_L(16);
+    }
+#undef SWL_DR_L
+    return SWL_ERR_UNSUPPORTED;
+}
+
+extern "C" int swl_gated_head_rmsnorm(void *out, const float *o, const void *gate, int64_t gate_stride, const float *w,
+                                      float eps, int64_t num_tokens, int32_t num_heads, int32_t vdim, int32_t dtype,
+                                      swl_stream_t stream) {
+    if (num_tokens < 0 || num_heads <= 0 || vdim <= 0 || gate_stride < static_cast<int64_t>(num_heads) * vdim)
+        return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!out || !o || !gate || !w) return SWL_ERR_BAD_ARG;
+    if (num_tokens > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::gated_head_rmsnorm_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), static_cast<T *>(out), o, static_cast<const T *>(gate),
+                           gate_stride, w, eps, num_heads, vdim);
+    });
+    return swl::check_launch();
+}

@@ -57,7 +57,7 @@ __device__ __forceinline__ float lane_dot2(const T *x, const T *w, int n, int la
 template <typename T>
 __global__ __launch_bounds__(kMoeThreads) void moe_route_kernel(int32_t *idx_out, float *w_out, const T *h,
                                                                 const float *router, const float *bias, int width,
-                                                                int experts, int top) {
+                                                                int experts, int top, int all_scores, float scale) {
     extern __shared__ float lds[];
     float *hf = lds;                // [width]
     float *logit = lds + width;     // [experts]
@@ -70,10 +70,18 @@ __global__ __launch_bounds__(kMoeThreads) void moe_route_kernel(int32_t *idx_out
         float a = 0.f;
         for (int i = lane; i < width; i += 64) a += hf[i] * wr[i];
         a = wave_allreduce_sum(a);
-        if (lane == 0) logit[e] = a + bias[e];
+        if (lane == 0) logit[e] = a + (bias ? bias[e] : 0.f);
     }
     __syncthreads();
     if (wave != 0) return;
+    // all_scores: the weights are scale * softmax over ALL experts (not renormalised over the chosen ones)
+    float all_max = -INFINITY, all_den = 0.f;
+    if (all_scores) {
+        for (int e = lane; e < experts; e += 64) all_max = fmaxf(all_max, logit[e]);
+        all_max = wave_allreduce_max(all_max);
+        for (int e = lane; e < experts; e += 64) all_den += expf(logit[e] - all_max);
+        all_den = wave_allreduce_sum(all_den);
+    }
     // top-k by repeated arg-max over the wave (each lane scans experts lane, lane + 64, ...)
     float chosen_max = 0.f, denom = 0.f;
     for (int j = 0; j < top; ++j) {
@@ -95,7 +103,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_route_kernel(int32_t *idx_out
                 besti = oi;
             }
         }
-        if (j == 0) chosen_max = best;
+        if (j == 0) chosen_max = all_scores ? all_max : best;
         const float pj = expf(best - chosen_max);
         denom += pj;
         if (lane == 0) {
@@ -106,8 +114,10 @@ __global__ __launch_bounds__(kMoeThreads) void moe_route_kernel(int32_t *idx_out
         __builtin_amdgcn_wave_barrier();
         __threadfence_block();
     }
-    if (lane == 0)
-        for (int j = 0; j < top; ++j) w_out[t * top + j] /= denom;
+    if (lane == 0) {
+        const float mult = all_scores ? scale / all_den : 1.0f / denom;
+        for (int j = 0; j < top; ++j) w_out[t * top + j] *= mult;
+    }
 }
 
 // grid (assignments, ceil(ff / 64)): wave w of the workgroup computes ff rows f0 + w, f0 + w + 4, ...
@@ -138,6 +148,39 @@ __global__ __launch_bounds__(kMoeThreads) void moe_gate_up_kernel(T *y, const T 
             y[a * ff + f] = to_t<T>(g * sg * (u + 1.0f));
         }
     }
+}
+
+// Experts without a gate: y = relu(W_up h)^2 for every (token, chosen expert); up [experts, ff, width]. Same grid.
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void moe_up_relu2_kernel(T *y, const T *h, const T *up, const int32_t *expert_idx,
+                                                                   int width, int ff, int top) {
+    extern __shared__ float lds[];
+    float *hf = lds;    // [width]
+    const int64_t a = blockIdx.x;
+    const int64_t t = a / top;
+    const int e = expert_idx[a];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int i = threadIdx.x; i < width; i += kMoeThreads) hf[i] = to_f(h[t * width + i]);
+    __syncthreads();
+    const T *wu = up + static_cast<int64_t>(e) * ff * width;
+    const int f0 = blockIdx.y * 64;
+    for (int f = f0 + wave; f < min(ff, f0 + 64); f += kMoeWaves) {
+        float u = wave_allreduce_sum(lane_dot(hf, wu + static_cast<int64_t>(f) * width, width, lane));
+        if (lane == 0) {
+            u = fmaxf(u, 0.f);
+            y[a * ff + f] = to_t<T>(u * u);
+        }
+    }
+}
+
+// y[r][f] = relu(z[r][f])^2 over rows of z that may be wider than ff (in_stride)
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void relu_sq_kernel(T *y, const T *z, int64_t total, int ff, int64_t in_stride) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kMoeThreads + threadIdx.x;
+    if (i >= total) return;
+    const int64_t r = i / ff;
+    const float v = fmaxf(to_f(z[r * in_stride + (i - r * ff)]), 0.f);
+    y[i] = to_t<T>(v * v);
 }
 
 // grid (tokens, ceil(width / 64)): wave w computes output columns c0 + w, c0 + w + 4, ...
@@ -174,13 +217,16 @@ constexpr int kEsRows = 64;         // outputs per workgroup at most (16 per wav
 constexpr int kEsTiles = 4;         // tiles of 16 assignments per pass over the weights
 constexpr int kEsMaxAssign = 1024;  // assignments per step (the sorted library path serves larger steps)
 
-template <typename T, bool GLU>
+template <typename T, int MODE>
 __global__ __launch_bounds__(kMoeThreads, 2) void moe_expert_stationary_kernel(T *out, const T *x, const T *w,
                                                                             const int32_t *expert_idx, int assignments,
                                                                             int K, int N, int top, float limit, int ksplit) {
     // ksplit = 1: every wave of the workgroup owns 16 outputs and the whole reduction. ksplit = waves of the workgroup: all
     // waves own the SAME 16 outputs and a quarter (half) of the reduction each; their accumulators meet in LDS and wave 0
     // finishes (short reductions and few outputs would otherwise leave most of the chip idle in a decode step).
+    // MODE 0: plain product, X rows are assignments; 1: clamped gated unit, X rows are tokens; 2: squared ReLU of the plain
+    // product (experts without a gate), X rows are tokens
+    constexpr bool GLU = MODE == 1;
     __shared__ int mine[kEsMaxAssign];
     __shared__ int count;
     __shared__ float red[3][2 * kEsTiles][256];
@@ -212,7 +258,7 @@ __global__ __launch_bounds__(kMoeThreads, 2) void moe_expert_stationary_kernel(T
             const int i = pass + t * 16 + li;
             const int a = i < m ? mine[i] : -1;
             arow[t] = a;
-            xp[t] = x + static_cast<int64_t>(a < 0 ? 0 : (GLU ? a / top : a)) * K + 8 * lq;
+            xp[t] = x + static_cast<int64_t>(a < 0 ? 0 : (MODE != 0 ? a / top : a)) * K + 8 * lq;
         }
         float4_t accg[kEsTiles], accu[kEsTiles];
 #pragma unroll
@@ -299,6 +345,10 @@ __global__ __launch_bounds__(kMoeThreads, 2) void moe_expert_stationary_kernel(T
                             const float u = fminf(fmaxf(accu[t][r], -limit), limit);
                             v = g * (1.0f / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
                         }
+                        if constexpr (MODE == 2) {
+                            v = fmaxf(v, 0.f);
+                            v *= v;
+                        }
                         out[static_cast<int64_t>(arow[t]) * N + n] = to_t<T>(v);
                     }
                 }
@@ -362,12 +412,16 @@ extern "C" int swl_moe_expert_stationary(void *out, const void *x, const void *w
     if (grid.y > 65535) return SWL_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     SWL_DISPATCH_DTYPE(dtype, T, {
-        if (glu)
-            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, true>), grid, dim3(64 * nw), lds, s,
+        if (glu == 1)
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, 1>), grid, dim3(64 * nw), lds, s,
+                               static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
+                               assignments, K, N, top, limit, ksplit);
+        else if (glu == 2)
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, 2>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
                                assignments, K, N, top, limit, ksplit);
         else
-            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, false>), grid, dim3(64 * nw), lds, s,
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, 0>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
                                assignments, K, N, top, limit, ksplit);
     });
@@ -415,7 +469,23 @@ extern "C" int swl_moe_route(int32_t *idx_out, float *w_out, const void *h, cons
     SWL_DISPATCH_DTYPE3(dtype, T, {
         hipLaunchKernelGGL((swl::moe_route_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kMoeThreads),
                            lds, static_cast<hipStream_t>(stream), idx_out, w_out, static_cast<const T *>(h), router, bias,
-                           width, experts, top);
+                           width, experts, top, 0, 1.0f);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_moe_route_scores(int32_t *idx_out, float *w_out, const void *h, const float *router, const float *bias,
+                                    int64_t num_tokens, int32_t width, int32_t experts, int32_t top, float scale,
+                                    int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || experts <= 0 || top <= 0 || top > experts) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!idx_out || !w_out || !h || !router) return SWL_ERR_BAD_ARG;
+    const size_t lds = (static_cast<size_t>(width) + experts) * 4;
+    if (num_tokens > 0x7fffffffLL || lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::moe_route_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kMoeThreads),
+                           lds, static_cast<hipStream_t>(stream), idx_out, w_out, static_cast<const T *>(h), router, bias,
+                           width, experts, top, 1, scale);
     });
     return swl::check_launch();
 }
@@ -450,6 +520,39 @@ extern "C" int swl_moe_down_combine(void *out, const void *y, const void *down, 
         hipLaunchKernelGGL((swl::moe_down_combine_kernel<T>), grid, dim3(swl::kMoeThreads), 0,
                            static_cast<hipStream_t>(stream), static_cast<T *>(out), static_cast<const T *>(y),
                            static_cast<const T *>(down), expert_idx, expert_w, width, ff, top);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_moe_up_relu2(void *y, const void *h, const void *up, const int32_t *expert_idx, int64_t num_tokens,
+                                int32_t width, int32_t ff, int32_t top, int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || ff <= 0 || top <= 0) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!y || !h || !up || !expert_idx) return SWL_ERR_BAD_ARG;
+    const size_t lds = static_cast<size_t>(width) * 4;
+    const int64_t assignments = num_tokens * top;
+    if (assignments > 0x7fffffffLL || lds > 64 * 1024 || (ff + 63) / 64 > 65535) return SWL_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(assignments), static_cast<unsigned>((ff + 63) / 64));
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::moe_up_relu2_kernel<T>), grid, dim3(swl::kMoeThreads), lds,
+                           static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(h),
+                           static_cast<const T *>(up), expert_idx, width, ff, top);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_relu_sq(void *y, const void *z, int64_t num_rows, int32_t ff, int64_t in_stride, int32_t dtype,
+                           swl_stream_t stream) {
+    if (num_rows < 0 || ff <= 0 || in_stride < ff) return SWL_ERR_BAD_ARG;
+    if (num_rows == 0) return SWL_OK;
+    if (!y || !z) return SWL_ERR_BAD_ARG;
+    const int64_t total = num_rows * ff;
+    const int64_t blocks = (total + swl::kMoeThreads - 1) / swl::kMoeThreads;
+    if (blocks > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::relu_sq_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(swl::kMoeThreads), 0,
+                           static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(z), total, ff,
+                           in_stride);
     });
     return swl::check_launch();
 }

@@ -90,6 +90,64 @@ __global__ __launch_bounds__(kQkThreads) void qknorm_store_kv_kernel(
     }
 }
 
+
+// The same store with ONE norm over the whole query projection and one over the whole key projection (all heads at once,
+// a weight per element), and a query multiplier that grows with the logarithm of the position:
+//   q <- q / rms(q) * q_w * (1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)).
+// store = 0: the row holds queries only (a layer that attends over another layer's keys and values).
+template <typename T>
+__global__ __launch_bounds__(kQkThreads) void qknorm_full_store_kv_kernel(
+    T *qkv, const float *q_w, const float *k_w, T *k_cache, T *v_cache, const int32_t *block_table,
+    const int32_t *tok_seq, const int32_t *tok_pos, int H, int G, int d, int dv, int64_t tok_stride,
+    int max_blocks_per_seq, int64_t block_stride, float eps, float temp_coef, int temp_every, int store) {
+    __shared__ float red[2][kQkThreads / 64];
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    T *row = qkv + t * tok_stride;
+    const int pos = tok_pos[t];
+    const int nq = H * d, nk = G * d;
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < nq; i += kQkThreads) {
+        const float v = to_f(row[i]);
+        sq += v * v;
+    }
+    if (store) {
+        for (int i = threadIdx.x; i < nk; i += kQkThreads) {
+            const float v = to_f(row[nq + i]);
+            sk += v * v;
+        }
+    }
+    sq = wave_allreduce_sum(sq);
+    sk = wave_allreduce_sum(sk);
+    if (lane == 0) {
+        red[0][wave] = sq;
+        red[1][wave] = sk;
+    }
+    __syncthreads();
+    sq = sk = 0.f;
+#pragma unroll
+    for (int w = 0; w < kQkThreads / 64; ++w) {
+        sq += red[0][w];
+        sk += red[1][w];
+    }
+    float rq = 1.0f / sqrtf(sq / static_cast<float>(nq) + eps);
+    if (temp_coef != 0.f) rq *= 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every + 1));
+    for (int i = threadIdx.x; i < nq; i += kQkThreads) row[i] = to_t<T>(to_f(row[i]) * q_w[i] * rq);
+    if (!store) return;
+    const float rk = 1.0f / sqrtf(sk / static_cast<float>(nk) + eps);
+    const int64_t blk = block_table[static_cast<int64_t>(tok_seq[t]) * max_blocks_per_seq + pos / kQkBlock];
+    const int off = pos % kQkBlock;
+    for (int i = threadIdx.x; i < nk; i += kQkThreads) {
+        const int g = i / d, e = i - g * d;
+        k_cache[blk * block_stride + (static_cast<int64_t>(g) * kQkBlock + off) * d + e] = to_t<T>(to_f(row[nq + i]) * k_w[i] * rk);
+    }
+    const T *vsrc = row + nq + nk;
+    for (int i = threadIdx.x; i < G * dv; i += kQkThreads) {
+        const int g = i / dv, c = i - g * dv;
+        v_cache[blk * block_stride + (static_cast<int64_t>(g) * dv + c) * kQkBlock + off] = vsrc[i];    // transposed page
+    }
+}
+
 } // namespace swl
 
 extern "C" int swl_qknorm_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_cache, void *v_cache,
@@ -110,6 +168,32 @@ extern "C" int swl_qknorm_store_kv(void *qkv, const float *q_w, const float *k_w
                            dim3(swl::kQkThreads), 0, static_cast<hipStream_t>(stream), static_cast<T *>(qkv), q_w, k_w,
                            static_cast<T *>(k_cache), static_cast<T *>(v_cache), block_table, tok_seq, tok_pos,
                            num_q_heads, num_kv_heads, dim, vdim, tok_stride, max_blocks_per_seq, block_stride, eps, store);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_qknorm_full_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_cache, void *v_cache,
+                                        const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                                        int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
+                                        int32_t vdim, int64_t tok_stride, int32_t max_blocks_per_seq,
+                                        int64_t block_stride, float eps, float temp_coef, int32_t temp_every,
+                                        int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || dim <= 0 || vdim <= 0 || temp_every < 1)
+        return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!qkv || !q_w || !tok_pos) return SWL_ERR_BAD_ARG;
+    const int store = k_cache != nullptr;
+    if (store && (!k_w || !v_cache || !block_table || !tok_seq)) return SWL_ERR_BAD_ARG;
+    const int64_t need = static_cast<int64_t>(num_q_heads) * dim +
+                         (store ? static_cast<int64_t>(num_kv_heads) * (dim + vdim) : 0);
+    if (tok_stride < need) return SWL_ERR_BAD_ARG;
+    if (num_tokens > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::qknorm_full_store_kv_kernel<T>), dim3(static_cast<unsigned>(num_tokens)),
+                           dim3(swl::kQkThreads), 0, static_cast<hipStream_t>(stream), static_cast<T *>(qkv), q_w, k_w,
+                           static_cast<T *>(k_cache), static_cast<T *>(v_cache), block_table, tok_seq, tok_pos,
+                           num_q_heads, num_kv_heads, dim, vdim, tok_stride, max_blocks_per_seq, block_stride, eps,
+                           temp_coef, temp_every, store);
     });
     return swl::check_launch();
 }

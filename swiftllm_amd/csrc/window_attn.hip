@@ -1,6 +1,7 @@
 // window_attn.hip — attention over the paged KV pool with a sliding window, tanh soft-capping and pre-softmax head
 // mixing ("talking heads": the capped scores of all query heads at one (query, key) pair are mixed by an [H, H] matrix
-// before the softmax), for any mixture of prompt portions and single decoded tokens.
+// before the softmax; without a matrix every head keeps its own) and an optional learned bias per (distance, head) added to
+// the mixed scores, for any mixture of prompt portions and single decoded tokens.
 //
 // Every query token carries its sequence row and position; its own key/value are already in the pool (qknorm_kv.hip ran
 // first), so a prompt portion that continues a cached prefix, a whole prompt and a decoded token are the same case:
@@ -30,8 +31,8 @@ __host__ __device__ inline size_t wa_float_count(int H, int d) {
 template <typename T>
 __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
-    const int32_t *tok_pos, const float *talk, int H, int G, int d, int dv, int64_t q_tok_stride, int window,
-    float scale, float softcap, int max_blocks_per_seq, int64_t block_stride) {
+    const int32_t *tok_pos, const float *talk, const float *rel, int rel_len, int H, int G, int d, int dv,
+    int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride) {
     extern __shared__ float lds[];
     float *qf = lds;                        // [H * d]
     float *tk = qf + H * d;                 // [H * H]
@@ -52,7 +53,8 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
 
     const T *qrow = q + t * q_tok_stride;
     for (int i = tid; i < H * d; i += kWaThreads) qf[i] = to_f(qrow[i]);
-    for (int i = tid; i < H * H; i += kWaThreads) tk[i] = talk[i];
+    // (no mixing matrix: every head keeps its own scores)
+    for (int i = tid; i < H * H; i += kWaThreads) tk[i] = talk ? talk[i] : (i / H == i % H ? 1.f : 0.f);
 
     float acc[kWaMaxAcc];
 #pragma unroll
@@ -98,7 +100,13 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
             float mixed = kNegBig;
             if (lane < cn) {
                 float a = 0.f;
-                for (int g = 0; g < H; ++g) a += tk[h * H + g] * s[g * kWaChunk + lane];
+                if (talk) {
+                    for (int g = 0; g < H; ++g) a += tk[h * H + g] * s[g * kWaChunk + lane];
+                } else {
+                    a = s[h * kWaChunk + lane];
+                }
+                // learned bias by distance (query position - key position), one row of the table per head
+                if (rel) a += rel[static_cast<int64_t>(h) * rel_len + min(nkeys - 1 - (c0 + lane), rel_len - 1)];
                 mixed = a;
             }
             const float cmax = wave_allreduce_max(mixed);
@@ -152,7 +160,8 @@ inline size_t wa_lds_bytes(int H, int d) {
 
 extern "C" int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v_cache,
                                const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
-                               const float *talk, int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads,
+                               const float *talk, const float *rel, int32_t rel_len, int64_t num_tokens,
+                               int32_t num_q_heads, int32_t num_kv_heads,
                                int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window, float scale,
                                float softcap, int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
                                swl_stream_t stream) {
@@ -160,7 +169,8 @@ extern "C" int swl_window_attn(void *out, const void *q, const void *k_cache, co
         return SWL_ERR_BAD_ARG;
     if (num_q_heads % num_kv_heads) return SWL_ERR_BAD_ARG;
     if (num_tokens == 0) return SWL_OK;
-    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !talk) return SWL_ERR_BAD_ARG;
+    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || (rel && rel_len <= 0))
+        return SWL_ERR_BAD_ARG;
     const size_t lds = swl::wa_lds_bytes(num_q_heads, dim);
     if (num_tokens > 0x7fffffffLL || num_q_heads > 32 ||
         static_cast<int64_t>(num_q_heads) * vdim > swl::kWaMaxAcc * swl::kWaThreads || lds > 64 * 1024)
@@ -169,7 +179,8 @@ extern "C" int swl_window_attn(void *out, const void *q, const void *k_cache, co
         hipLaunchKernelGGL((swl::window_attn_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kWaThreads),
                            lds, static_cast<hipStream_t>(stream), static_cast<T *>(out), static_cast<const T *>(q),
                            static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, tok_seq,
-                           tok_pos, talk, num_q_heads, num_kv_heads, dim, vdim, q_tok_stride, window, scale, softcap,
+                           tok_pos, talk, rel, rel_len, num_q_heads, num_kv_heads, dim, vdim, q_tok_stride, window, scale,
+                           softcap,
                            max_blocks_per_seq, block_stride);
     });
     return swl::check_launch();

@@ -22,7 +22,8 @@ constexpr int kWmTile = 16;     // queries per tile = keys per page = MFMA edge
 template <typename T, int D, int DV, int HPW, int NW>
 __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
-    const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk, int H, int G,
+    const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk,
+    const float *__restrict__ rel, int rel_len, int H, int G,
     int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
     float *part_o, float *part_ml, int64_t num_tokens, int nbuf) {
     // [nbuf][H][64 lanes][4] capped scores of a page, then [H][H] the mixing matrix. nbuf = 2: pages alternate between two
@@ -37,7 +38,8 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // (tells the compiler that it is wave-uniform)
     const int li = lane & 15, lq = lane >> 4;       // query (or operand row) index; quarter
-    for (int i = tid; i < H * H; i += NW * 64) tk[i] = talk[i] * kLog2e;     // mixed scores come out in base-2 exponent units
+    // mixed scores come out in base-2 exponent units; without a matrix every head keeps its own scores
+    for (int i = tid; i < H * H; i += NW * 64) tk[i] = talk ? talk[i] * kLog2e : (i / H == i % H ? kLog2e : 0.f);
     __syncthreads();
     const int p0 = __builtin_amdgcn_readfirstlane(tok_pos[row0]);
     const int32_t *bt = block_table + static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tok_seq[row0])) * max_blocks_per_seq;
@@ -179,6 +181,15 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
                 for (int r = 0; r < 4; ++r) mixed[hh][r] += tw * sv[r];
             }
         }
+        if (rel) {      // learned bias by distance (query position - key position), one row of the table per head
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const float *rh = rel + static_cast<int64_t>(min(h0 + hh, H - 1)) * rel_len;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    mixed[hh][r] += rh[min(max(qpos - (kpos0 + r), 0), rel_len - 1)] * kLog2e;
+            }
+        }
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int h = h0 + hh;
@@ -281,11 +292,12 @@ __global__ __launch_bounds__(256) void window_attn_combine_kernel(T *out, const 
 template <typename T, int D, int DV>
 int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q, const T *kc, const T *vc,
               const int32_t *bt, const int32_t *ts, const int32_t *tp, const int32_t *r0, const int32_t *cn,
-              const float *talk, int H, int G, int64_t qs, int window, float scale, float softcap, int mb, int64_t bs,
+              const float *talk, const float *rel, int rel_len, int H, int G, int64_t qs, int window, float scale,
+              float softcap, int mb, int64_t bs,
               float *po, float *pml, int64_t nt, int nbuf) {
 #define SWL_WM_LAUNCH(HPW, NW)                                                                                          \
     hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW, NW>), grid, dim3(NW * 64), lds, s, out, q, kc, vc, bt, ts, \
-                       tp, r0, cn, talk, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf)
+                       tp, r0, cn, talk, rel, rel_len, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf)
     // heads per wave x waves: up to 16 heads on four waves, more on eight (four heads per wave at most: the accumulators of
     // eight 128-wide heads do not fit a wave's registers)
     switch (hpw) {
@@ -318,7 +330,7 @@ extern "C" int swl_window_attn_tiles_supported(int32_t num_q_heads, int32_t num_
 extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache,
                                      const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
                                      const int32_t *tile_row0, const int32_t *tile_cnt, const float *talk,
-                                     int32_t num_tiles, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
+                                     const float *rel, int32_t rel_len, int32_t num_tiles, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
                                      int32_t vdim, int64_t q_tok_stride, int32_t window, float scale, float softcap,
                                      int32_t max_blocks_per_seq, int64_t block_stride, int32_t key_splits,
                                      float *scratch, int64_t num_tokens, int32_t dtype, swl_stream_t stream) {
@@ -327,7 +339,8 @@ extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cac
         return SWL_ERR_BAD_ARG;
     if (!swl_window_attn_tiles_supported(num_q_heads, num_kv_heads, dim, vdim, dtype)) return SWL_ERR_UNSUPPORTED;
     if (num_tiles == 0) return SWL_OK;
-    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !tile_row0 || !tile_cnt || !talk)
+    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !tile_row0 || !tile_cnt ||
+        (rel && rel_len <= 0))
         return SWL_ERR_BAD_ARG;
     if ((q_tok_stride & 3) || (block_stride & 3) || (reinterpret_cast<uintptr_t>(q) & 7) ||
         (reinterpret_cast<uintptr_t>(k_cache) & 7) || (reinterpret_cast<uintptr_t>(out) & 7))
@@ -346,7 +359,7 @@ extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cac
     if (dim == DD && vdim == DDV)                                                                                         \
         return swl::launch_wm<T, DD, DDV>(hpw, grid, lds, s, static_cast<T *>(out), static_cast<const T *>(q),           \
                                           static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, \
-                                          tok_seq, tok_pos, tile_row0, tile_cnt, talk, num_q_heads, num_kv_heads,        \
+                                          tok_seq, tok_pos, tile_row0, tile_cnt, talk, rel, rel_len, num_q_heads, num_kv_heads, \
                                           q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride, part_o, \
                                           part_ml, num_tokens, nbuf);
     SWL_DISPATCH_DTYPE(dtype, T, {

@@ -157,3 +157,173 @@ class KekapelModelConfig:
     def load_from_model_path(model_path: str) -> "KekapelModelConfig":
         with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
             return KekapelModelConfig(json.load(f))
+
+
+# ---- Lorulix ---------------------------------------------------------------------------------------------------------------
+def distance_bias_rows(table_rows: int, far: float, max_distance: int):
+    """Row of a learned distance-bias table for every distance 0 .. max_distance - 1: the first table_rows // 2 distances have
+    a row each, beyond that the rows advance in equal steps of log(distance) and the last row is reached at `far`."""
+    import math
+    half = table_rows // 2
+    rows = []
+    for dist in range(max_distance):
+        if dist < half:
+            rows.append(dist)
+        else:
+            rows.append(min(table_rows - 1,
+                            half + int(math.floor(math.log(dist / half) / math.log(far / half) * (table_rows - half)))))
+    return rows
+
+
+class LorulixAttentionConfig:
+    """Softmax attention over every earlier key with a whole-projection q/k RMS norm, a position-dependent query
+    temperature and a learned bias per (distance bucket, head); optionally on another layer's keys and values."""
+    kind = "attention"
+
+    def __init__(self, mixer: dict):
+        self.num_q_heads = int(mixer["heads"])
+        self.num_kv_heads = int(mixer.get("kv_heads", self.num_q_heads))
+        self.head_dim = int(mixer["dim"])
+        self.value_dim = int(mixer.get("vdim", self.head_dim))
+        self.scale = float(mixer["scale"])
+        self.softcap = 0.0
+        self.window = 0
+        self.bias_max = float(mixer["bias_max"]) if mixer.get("bias_max") else 0.0     # 0: no distance bias
+        temp = mixer.get("q_temp") or {}
+        self.q_temp_coef = float(temp.get("coef", 0.0))
+        self.q_temp_every = int(temp.get("every", 1))
+        self.kv_from = int(mixer["kv_from"]) if mixer.get("kv_from") is not None else -1     # -1: its own keys and values
+        if self.num_q_heads % self.num_kv_heads:
+            raise ValueError(f"heads ({self.num_q_heads}) must be a multiple of kv_heads ({self.num_kv_heads})")
+        if self.q_temp_every < 1:
+            raise ValueError(f"q_temp.every must be positive, got {self.q_temp_every}")
+
+    @property
+    def q_size(self) -> int:
+        return self.num_q_heads * self.head_dim
+
+    @property
+    def k_size(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def v_size(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+
+class LorulixDeltaConfig:
+    """Gated delta rule: a [dim, vdim] fp32 state per head, short causal convolutions on q, k and v."""
+    kind = "delta"
+
+    def __init__(self, mixer: dict):
+        self.num_heads = int(mixer["heads"])
+        self.num_kv_heads = int(mixer.get("kv_heads", self.num_heads))      # q/k heads
+        self.head_dim = int(mixer["dim"])
+        self.value_dim = int(mixer.get("vdim", self.head_dim))
+        self.conv_taps = int(mixer.get("conv", 1))
+        if self.num_heads % self.num_kv_heads:
+            raise ValueError(f"heads ({self.num_heads}) must be a multiple of kv_heads ({self.num_kv_heads})")
+        if self.conv_taps < 1:
+            raise ValueError(f"conv must be positive, got {self.conv_taps}")
+
+    @property
+    def qk_size(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def v_size(self) -> int:
+        return self.num_heads * self.value_dim
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.qk_size + self.v_size
+
+    @property
+    def proj_size(self) -> int:
+        """Rows of the fused input projection: q | k | v | output gate | beta | decay."""
+        return 2 * self.qk_size + 2 * self.v_size + 2 * self.num_heads
+
+    @property
+    def state_elems(self) -> int:
+        return self.num_heads * self.head_dim * self.value_dim
+
+
+class LorulixMlpConfig:
+    """`dense`: clamped gated unit. `moe`: softmax router over all experts, squared-ReLU experts, optional shared expert."""
+
+    def __init__(self, mlp: dict):
+        self.kind = mlp["kind"]
+        self.shared_ffn_inter_dim = 0
+        if self.kind == "dense":
+            self.ffn_inter_dim = int(mlp["ff"])
+            self.limit = float(mlp["limit"])
+        elif self.kind == "moe":
+            self.ffn_inter_dim = int(mlp["expert"]["ff"])
+            self.num_experts = int(mlp["router"]["experts"])
+            self.top_k = int(mlp["router"]["top"])
+            self.router_scale = float(mlp["router"].get("scale", 1.0))
+            if mlp.get("shared"):
+                self.shared_ffn_inter_dim = int(mlp["shared"]["ff"])
+            if not 0 < self.top_k <= self.num_experts:
+                raise ValueError(f"router.top ({self.top_k}) must be in 1..experts ({self.num_experts})")
+        else:
+            raise ValueError(f"unsupported mlp.kind {self.kind!r}")
+
+
+class LorulixLayerConfig:
+    def __init__(self, layer: dict):
+        self.type = layer["type"]
+        if self.type == "attention":
+            self.mixer = LorulixAttentionConfig(layer["mixer"])
+        elif self.type == "delta":
+            self.mixer = LorulixDeltaConfig(layer["mixer"])
+        else:
+            raise ValueError(f"unsupported layer type {self.type!r}")
+        self.mlp = LorulixMlpConfig(layer["mlp"]) if layer.get("mlp") else None
+
+
+class LorulixModelConfig:
+    """Lorulix: a decoder-only model with learned positions and an fp32 stream; every sublayer reads the RMS-normed stream
+    plus a short causal convolution of it, and its result is gated, normed and added. Mixers are gated-delta-rule
+    recurrences or distance-biased softmax attention (possibly on an earlier layer's keys and values); feed-forwards are a
+    clamped gated unit or a mixture of squared-ReLU experts. Every size and constant is read from config.json."""
+
+    def __init__(self, model_config: dict):
+        if model_config.get("architecture") != "Lorulix":
+            raise AssertionError(f"unsupported architecture {model_config.get('architecture')!r}")
+        self.vocab_size = int(model_config["vocab"])
+        self.hidden_size = int(model_config["width"])
+        self.max_position_embeddings = int(model_config["max_positions"])
+        self.norm_eps = float(model_config["norm"]["eps"])
+        self.canon_taps = int((model_config.get("canon") or {}).get("taps", 1))
+        if self.canon_taps < 1:
+            raise ValueError(f"canon.taps must be positive, got {self.canon_taps}")
+        self.layers = [LorulixLayerConfig(layer) for layer in model_config["layers"]]
+        self.num_layers = len(self.layers)
+        for i, layer in enumerate(self.layers):
+            if layer.type != "attention" or layer.mixer.kv_from < 0:
+                continue
+            j = layer.mixer.kv_from
+            src = self.layers[j] if 0 <= j < i else None
+            if src is None or src.type != "attention" or src.mixer.kv_from >= 0:
+                raise ValueError(f"layer {i}: kv_from {j} must name an earlier attention layer with keys of its own")
+            a, b = layer.mixer, src.mixer
+            if (a.num_kv_heads, a.head_dim, a.value_dim) != (b.num_kv_heads, b.head_dim, b.value_dim):
+                raise ValueError(f"layer {i}: key/value sizes differ from those of layer {j}")
+        attn = [l.mixer for l in self.layers if l.type == "attention"] or [None]
+        # what the scheduler-facing code reads off any model's configuration
+        self.num_q_heads = max((m.num_q_heads for m in attn if m), default=1)
+        self.num_kv_heads = max((m.num_kv_heads for m in attn if m), default=1)
+        self.head_dim = max((m.head_dim for m in attn if m), default=1)
+
+    def kv_elems_per_token(self) -> int:
+        """K and V elements one token occupies over the attention layers that keep their own."""
+        return sum(l.mixer.k_size + l.mixer.v_size for l in self.layers if l.type == "attention" and l.mixer.kv_from < 0)
+
+    def get_kvslot_size(self, dtype: torch.dtype = torch.bfloat16) -> int:
+        return max(self.kv_elems_per_token(), 1) * dtype.itemsize
+
+    @staticmethod
+    def load_from_model_path(model_path: str) -> "LorulixModelConfig":
+        with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
+            return LorulixModelConfig(json.load(f))

@@ -12,6 +12,7 @@ import os
 MODELS = {
     "llama": ("swiftllm_amd.model_config:LlamaModelConfig", "swiftllm_amd.worker.model:LlamaModel"),
     "Kekapel": ("swiftllm_amd.model_config:KekapelModelConfig", "swiftllm_amd.worker.kekapel_model:KekapelModel"),
+    "Lorulix": ("swiftllm_amd.model_config:LorulixModelConfig", "swiftllm_amd.worker.lorulix_model:LorulixModel"),
 }
 
 

@@ -160,9 +160,16 @@ class StepPlan:
     # tiles of up to TILE consecutive tokens of one sequence (the matrix-core attention's unit of work)
     tile_row0: np.ndarray = None        # [NT] int32 first token row of each tile
     tile_cnt: np.ndarray = None         # [NT] int32 tokens in it
+    # the portions themselves (what recurrent layers walk token by token) and, per token, where its portion starts
+    seq_row0: np.ndarray = None         # [S] int32 first token row of each sequence's portion
+    seq_cnt: np.ndarray = None          # [S] int32 tokens in it
+    tok_start: np.ndarray = None        # [T] int32 position of the first token of the token's portion
+    # [T] int32 state slot * 2 + tail parity of the token's sequence; zeros until a worker with per-sequence state fills it
+    tok_state: np.ndarray = None
 
     TILE = 16
-    SEGMENTS = ("input_ids", "tok_pos", "tok_seq", "want_rows", "tile_row0", "tile_cnt")
+    SEGMENTS = ("input_ids", "tok_pos", "tok_seq", "want_rows", "tile_row0", "tile_cnt", "seq_row0", "seq_cnt", "tok_start",
+                "tok_state")
 
     def packed_layout(self):
         out, off = [], 0
@@ -216,6 +223,10 @@ def plan_step(entries: Sequence[StepEntry], vocab_size: int = None, max_position
         row0.append(at + starts)
         cnt.append(np.minimum(StepPlan.TILE, n - starts).astype(np.int32))
         at += n
-    return StepPlan(tile_row0=cat(row0), tile_cnt=cat(cnt),
+    counts = np.asarray([len(e.tokens) for e in entries], dtype=np.int32)
+    starts = np.asarray([e.start for e in entries], dtype=np.int32)
+    return StepPlan(tile_row0=cat(row0), tile_cnt=cat(cnt), seq_cnt=counts,
+                    seq_row0=(np.cumsum(counts) - counts).astype(np.int32), tok_start=np.repeat(starts, counts),
+                    tok_state=np.zeros(base, dtype=np.int32),
                     num_tokens=base, num_seqs=len(seq_ids), seq_ids_list=seq_ids, target_lens_list=targets,
                     input_ids=cat(ids), tok_pos=cat(pos), tok_seq=cat(seq), want_rows=np.asarray(want, dtype=np.int32))

@@ -1,43 +1,25 @@
 """KekapelModel — the data-plane worker for the Kekapel design.
 
-Same worker protocol as LlamaModel (the Engine, the scheduler and the examples drive either):
-
-    model = KekapelModel(engine_config); model.load_weights()
-    n = model.profile_num_blocks(); model.init_kvcache_and_swap(n)
-    tokens = model.forward(input_ids_list, seq_ids_list, decoding_seq_lens_list)
-    model.swap_in_seqs(ids) / model.swap_out_seqs(ids) / model.free_seqs_resources(ids)
-
-plus the more general `step(entries)`, which `forward` is built on: every sequence brings a PORTION of tokens that
-continues it at a given position — a whole prompt, a slice of one, or one decoded token — and all portions of a step run
-as one batch. The kernels are token-level (each token carries its block-table row and position), so nothing distinguishes
-a prompt slice with a cached prefix from a decoded token.
-
-State: ONE block pool [num_blocks, elements per block] in the compute dtype. A 16-token block holds, side by side, the
-keys and values of every LAYER RUN (a layer inside the loop runs several times with the same weights and has a separate
-slice per pass); the block table and the allocator are the framework's BlockManager, shared by all runs. The residual
-stream is fp32; projections run in the compute dtype (bfloat16 / float16, or true float32).
+The worker protocol, the token-level `step`, the block pool, the block managers, hipGraph replay of decode steps and
+swapping are SteppedModel's (stepped_model.py); this file adds what is Kekapel's: the layout of a block (a 16-token block
+holds, side by side, the keys and values of every LAYER RUN — a layer inside the loop runs several times with the same
+weights and has a separate slice per pass), the weights, and the stack: embedding, sandwich LayerNorms fused with the fp32
+stream update, attention and feed-forward sublayers, the loop's pass additions. Projections run in the compute dtype
+(bfloat16 / float16, or true float32).
 """
-import math
-from typing import List, Sequence
+from typing import List
 
 import torch
 
-from swiftllm_amd import _hip
 from swiftllm_amd.engine_config import EngineConfig
 from swiftllm_amd.model_config import KekapelModelConfig
-from swiftllm_amd.utils import GB
 
-from .batch_plan import StepEntry, StepPlan, plan_step
-from .block_manager import BlockManager
 from .kekapel_weight import load_kekapel_weights
-from .kernels.block_swapping import swap_blocks
 from .kernels.layernorm import add_layernorm, embed_positions, layernorm
 from .kernels.linear import pack_weight, packable
-from .kernels.sampling import argmax_rows
 from .kernels.window_attn import PoolSlice
 from .layers.kekapel_layer import KekapelAttention, KekapelFeedForward, _project
-
-_DTYPES = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32}
+from .stepped_model import SteppedModel
 
 
 class _Sublayer:
@@ -45,35 +27,14 @@ class _Sublayer:
     __slots__ = ("kind", "run", "op", "pre", "post", "pass_index", "ends_run")
 
 
-class KekapelModel:
-    SUPPORTED_DTYPES = tuple(_DTYPES)
+class KekapelModel(SteppedModel):
+    CONFIG_CLASS = KekapelModelConfig
 
     @torch.inference_mode()
     def __init__(self, engine_config: EngineConfig):
-        self.engine_config = engine_config
-        self.model_config = KekapelModelConfig.load_from_model_path(engine_config.model_path)
-        self.dtype = _DTYPES[getattr(engine_config, "dtype", "bfloat16")]
-        self.device = torch.device("cuda")
-        self.weight = None
         self.sublayers: List[_Sublayer] = []
-        self.num_blocks = None
-        self.kv_pool = self.kv_swap = None
-        self.gpu_block_manager = self.cpu_block_manager = None
         self.pool_slices: List[PoolSlice] = []
-        self.block_elems = 0
-        self._layout_pool()
-        self._meta_host = self._meta_host_np = self._meta_dev = self._meta_done = None
-        self.after_launch_hook = None
-        # pure-decode steps (every sequence brings one token and asks for its logits) replay a captured hipGraph, one per
-        # batch size: the step's launch geometry depends on the token count only, never on positions or block ids
-        self._decode_graphs = {}
-        self._graph_pool = None
-        self.graph_captures = 0
-        # tests set these to lists: the fp32 stream after every layer run / the logits of every step
-        self.layer_tap = None
-        self.logits_tap = None
-        # what the scheduler asks any worker: how long a sequence may grow
-        self.max_seq_len = self.model_config.max_position_embeddings
+        super().__init__(engine_config)
 
     def _layout_pool(self):
         """Offsets (in elements) of every layer run's keys and values inside a block."""
@@ -88,15 +49,7 @@ class KekapelModel:
             off += mx.v_size * bs
         self.block_elems = off
 
-    # ---- set-up ------------------------------------------------------------------------------------------------------
-    @torch.inference_mode()
-    def load_weights(self):
-        if not torch.cuda.is_available():
-            raise _hip.HipLibraryError("no HIP device visible: swiftllm_amd's data plane runs only on an AMD GPU (gfx950)")
-        _hip.load()
-        if self.dtype == torch.float32:
-            torch.backends.cuda.matmul.allow_tf32 = False      # true fp32 products
-            torch.set_float32_matmul_precision("highest")
+    def _build(self):
         cfg, ecfg = self.model_config, self.engine_config
         self.weight = load_kekapel_weights(cfg, self.dtype, ecfg.model_path, ecfg.use_dummy, self.device)
         skinny = bool(getattr(ecfg, "use_skinny_gemm", False)) and self.dtype != torch.float32
@@ -119,68 +72,6 @@ class KekapelModel:
                 f.kind, f.run, f.op = "ff", run.index, KekapelFeedForward(lcfg, lw, eps, skinny)
                 f.pre, f.post, f.pass_index, f.ends_run = (lw.norm2_w, lw.norm2_b), (lw.norm2b_w, lw.norm2b_b), -1, True
                 self.sublayers.append(f)
-
-    @torch.inference_mode()
-    def profile_num_blocks(self) -> int:
-        """How many blocks fit: one forged worst-case step without a pool, the allocator's high-water mark, and the rest
-        of the usable memory divided by a block's bytes."""
-        ecfg = self.engine_config
-        torch.cuda.empty_cache()
-        torch.cuda.reset_peak_memory_stats()
-        num_tokens = min(ecfg.max_tokens_in_batch, ecfg.max_batch_size * self.model_config.max_position_embeddings)
-        batch = min(ecfg.max_batch_size, num_tokens)
-        lens = [num_tokens // batch] * batch
-        lens[-1] += num_tokens % batch
-        saved = self.kv_pool
-        self.kv_pool = None
-        self.forward([[0] * n for n in lens], list(range(batch)), [], ignore_kvcache=True)
-        self.kv_pool = saved
-        torch.cuda.synchronize()
-        free_memory, total_memory = torch.cuda.mem_get_info()
-        peak = total_memory - free_memory
-        usable = total_memory * ecfg.gpu_mem_utilization
-        print(f"[Model.profile] GPU total memory: {total_memory / GB:.2f} GB, runtime peak memory: {peak / GB:.2f} GB")
-        if usable < peak:
-            raise RuntimeError(f"Peak memory {peak / GB:.2f} GB exceeds usable memory {usable / GB:.2f} GB")
-        block_bytes = self.block_elems * self.dtype.itemsize
-        table_bytes = 2 * ecfg.max_seqs_in_block_table * ecfg.max_blocks_per_seq * 4
-        torch.cuda.empty_cache()
-        return max(math.floor((usable - peak - table_bytes) / block_bytes), 0)
-
-    @torch.inference_mode()
-    def init_kvcache_and_swap(self, num_blocks: int):
-        ecfg = self.engine_config
-        self.num_blocks = num_blocks
-        # zeros: a slot that was never written must not hold NaN bit patterns
-        self.kv_pool = torch.zeros((num_blocks, self.block_elems), dtype=self.dtype, device=self.device)
-        pin = getattr(ecfg, "pin_swap_memory", True) and ecfg.num_cpu_blocks > 0
-        try:
-            self.kv_swap = torch.zeros((ecfg.num_cpu_blocks, self.block_elems), dtype=self.dtype, pin_memory=pin)
-        except RuntimeError:
-            self.kv_swap = torch.zeros((ecfg.num_cpu_blocks, self.block_elems), dtype=self.dtype)
-        self._decode_graphs.clear()     # (captured against the previous pool and block table)
-        self._graph_pool = None
-        self.gpu_block_manager = BlockManager("GPU", num_blocks, ecfg.max_seqs_in_block_table, ecfg.max_blocks_per_seq,
-                                              ecfg.block_size, self.device)
-        self.cpu_block_manager = BlockManager("CPU", ecfg.num_cpu_blocks, ecfg.max_seqs_in_block_table,
-                                              ecfg.max_blocks_per_seq, ecfg.block_size, self.device)
-
-    # ---- one step ----------------------------------------------------------------------------------------------------
-    def _upload_plan(self, plan: StepPlan):
-        """The plan's int32 arrays through ONE pinned buffer and ONE async copy; returns device views."""
-        layout, total = plan.packed_layout()
-        if self._meta_done is not None:
-            self._meta_done.synchronize()
-        if self._meta_host is None or self._meta_host.numel() < total:
-            cap = max(total, 4 * self.engine_config.max_tokens_in_batch + 64)
-            self._meta_host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
-            self._meta_host_np = self._meta_host.numpy()
-            self._meta_dev = torch.empty(cap, dtype=torch.int32, device=self.device)
-            self._meta_done = torch.cuda.Event()
-        plan.pack_into(self._meta_host_np)
-        self._meta_dev[:total].copy_(self._meta_host[:total], non_blocking=True)
-        self._meta_done.record()
-        return {name: self._meta_dev[off:off + n] for name, off, n in layout}
 
     @torch.inference_mode()
     def _run_stack(self, dev: dict, use_pool: bool) -> torch.Tensor:
@@ -225,108 +116,3 @@ class KekapelModel:
         w = self.weight
         h = layernorm(x, w.final_norm_w, w.final_norm_b, self.model_config.norm_eps, self.dtype, rows)
         return _project(h, w.head, self._skinny)
-
-    @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry], ignore_kvcache: bool = False) -> torch.Tensor:
-        """Run one batch of portions. Returns the logits of the wanted places, [wanted, vocab] (device tensor in the compute
-        dtype), in the order of the entries and of each entry's `want`."""
-        cfg = self.model_config
-        plan = plan_step(entries, cfg.vocab_size, cfg.max_position_embeddings)
-        if plan.num_tokens == 0:
-            return torch.empty((0, cfg.vocab_size), dtype=self.dtype, device=self.device)
-        if not ignore_kvcache:
-            self.gpu_block_manager.allocate_blocks_for_seqs(plan.seq_ids_list, plan.target_lens_list)
-        dev = self._upload_plan(plan)
-        if (getattr(self.engine_config, "use_hip_graph", False) and not ignore_kvcache and self.layer_tap is None
-                and plan.num_tokens == plan.num_seqs == plan.want_rows.size):
-            logits = self._step_decode_graph(plan, dev)
-        else:
-            x = self._run_stack(dev, not ignore_kvcache)
-            if plan.want_rows.size == 0:
-                return torch.empty((0, cfg.vocab_size), dtype=self.dtype, device=self.device)
-            logits = self._logits(x, dev["want_rows"])
-        if self.logits_tap is not None:
-            self.logits_tap.append(logits.clone())
-        return logits
-
-    _MAX_DECODE_GRAPHS = 64
-
-    def _step_decode_graph(self, plan: StepPlan, dev: dict) -> torch.Tensor:
-        """Replay (capturing it first, once per batch size) the whole pure-decode step. The metadata buffer has a fixed
-        address and a layout that depends on the token count only, so a replay reads this step's tokens, positions and
-        block-table rows from where the capture did. The returned logits are the graph's own output buffer: valid until
-        the next replay of the same graph."""
-        key = plan.num_tokens
-        entry = self._decode_graphs.pop(key, None)
-        if entry is not None and entry[2] != self._meta_dev.data_ptr():
-            entry = None        # the metadata buffer was re-allocated: the capture points at the old one
-        if entry is None:
-            self.graph_captures += 1
-            warm = torch.cuda.Stream()      # one eager run first: nothing may be lazily initialised under capture
-            warm.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(warm):
-                self._logits(self._run_stack(dev, True), dev["want_rows"])
-            torch.cuda.current_stream().wait_stream(warm)
-            while len(self._decode_graphs) >= self._MAX_DECODE_GRAPHS:
-                self._decode_graphs.pop(next(iter(self._decode_graphs)))
-            if self._graph_pool is None:
-                self._graph_pool = torch.cuda.graph_pool_handle()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                out = self._logits(self._run_stack(dev, True), dev["want_rows"])
-            entry = (graph, out, self._meta_dev.data_ptr())
-        self._decode_graphs[key] = entry
-        entry[0].replay()
-        return entry[1]
-
-    @torch.inference_mode()
-    def forward(self, input_ids_list: List[List[int]], seq_ids_list: List[int], decoding_seq_lens_list: List[int],
-                ignore_kvcache: bool = False) -> List[int]:
-        """The worker protocol's iteration: whole prompts first, then decoding sequences (one token each, their lengths
-        INCLUDING it). Returns the greedy next token of every sequence."""
-        if len(input_ids_list) == 0:
-            return []
-        num_prefill = len(input_ids_list) - len(decoding_seq_lens_list)
-        if num_prefill < 0 or len(seq_ids_list) != len(input_ids_list):
-            raise ValueError("inconsistent batch: need len(seq_ids) == len(input_ids) >= len(decoding_seq_lens)")
-        entries = []
-        for i, (ids, sid) in enumerate(zip(input_ids_list, seq_ids_list)):
-            if i < num_prefill:
-                entries.append(StepEntry(sid, ids, 0, (len(ids) - 1,)))
-            else:
-                if len(ids) != 1:
-                    raise ValueError("every decoding sequence must contribute exactly one token")
-                entries.append(StepEntry(sid, ids, decoding_seq_lens_list[i - num_prefill] - 1, (0,)))
-        logits = self.step(entries, ignore_kvcache)
-        tokens = argmax_rows(logits)
-        if self.after_launch_hook is not None:
-            self.after_launch_hook()
-        return tokens.tolist()
-
-    # ---- swapping / release ------------------------------------------------------------------------------------------
-    def _swap(self, seq_ids_list: List[int], is_swap_in: bool):
-        if len(seq_ids_list) == 0:
-            return
-        src_mgr = self.cpu_block_manager if is_swap_in else self.gpu_block_manager
-        dst_mgr = self.gpu_block_manager if is_swap_in else self.cpu_block_manager
-        counts = src_mgr.get_num_allocated_blocks_host(seq_ids_list)
-        src_ids = [b for s in seq_ids_list for b in src_mgr.get_block_ids_host(s)]
-        src_mgr.gather_allocated_blocks_and_free(seq_ids_list)
-        dst_mgr.allocate_blocks_for_seqs(seq_ids_list, [c * self.engine_config.block_size for c in counts])
-        dst_ids = [b for s in seq_ids_list for b in dst_mgr.get_block_ids_host(s)]
-        swap_blocks(src_ids, dst_ids, is_swap_in, self.kv_pool, None, self.kv_swap, None)
-
-    @torch.inference_mode()
-    def swap_in_seqs(self, seq_ids_list: List[int]):
-        self._swap(seq_ids_list, True)
-
-    @torch.inference_mode()
-    def swap_out_seqs(self, seq_ids_list: List[int]):
-        self._swap(seq_ids_list, False)
-
-    @torch.inference_mode()
-    def free_seqs_resources(self, seq_ids_list: List[int]):
-        if len(seq_ids_list) == 0:
-            return
-        self.gpu_block_manager.free_blocks_for_seqs(seq_ids_list)
-        self.cpu_block_manager.free_blocks_for_seqs(seq_ids_list)

@@ -109,7 +109,7 @@ def _checkpoint_getter(model_path: str) -> Getter:
         if name not in table:
             raise KeyError(f"weight {name} not found in the checkpoint")
         path, st_dtype, st_shape, b, e = table[name]
-        if tuple(st_shape) != tuple(shape):
+        if len(st_shape) != len(shape) or any(b is not None and a != b for a, b in zip(st_shape, shape)):     # None: any size
             raise ValueError(f"shape of weight {name} does not match: {tuple(st_shape)} vs {tuple(shape)}")
         if st_dtype not in kinds:
             raise TypeError(f"weight {name}: unsupported dtype {st_dtype}")
@@ -117,7 +117,7 @@ def _checkpoint_getter(model_path: str) -> Getter:
         if path not in maps:
             maps[path] = np.memmap(path, dtype=np.uint8, mode="r")
         raw = torch.from_numpy(np.array(maps[path][b:e], copy=True))
-        return raw.view(tdtype).reshape(shape)
+        return raw.view(tdtype).reshape(tuple(st_shape))
     return get
 
 

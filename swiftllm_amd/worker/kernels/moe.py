@@ -19,6 +19,79 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top_k: 
     return idx, wts
 
 
+def moe_route_scores(h: torch.Tensor, router: torch.Tensor, top_k: int, scale: float):
+    """-> (expert ids int32 [T, top_k], weights fp32 [T, top_k]): the top_k experts by fp32 logit; weights = scale * softmax
+    over ALL experts at the chosen ones (not renormalised)."""
+    _hip.require_gpu_tensor(h, "h")
+    n, width = h.shape
+    experts = router.shape[0]
+    assert h.is_contiguous() and router.dtype == torch.float32 and router.is_contiguous() and router.shape[1] == width
+    idx = torch.empty((n, top_k), dtype=torch.int32, device=h.device)
+    wts = torch.empty((n, top_k), dtype=torch.float32, device=h.device)
+    _hip.call("swl_moe_route_scores", _hip.ptr(idx), _hip.ptr(wts), _hip.ptr(h), _hip.ptr(router), 0, n, width, experts,
+              top_k, float(scale), _hip.dtype_code3(h.dtype), _hip.stream())
+    return idx, wts
+
+
+def relu_squared(z: torch.Tensor, ff: int) -> torch.Tensor:
+    """relu(z[:, :ff])^2 -> [rows, ff] (z may have more columns)."""
+    assert z.dim() == 2 and z.stride(1) == 1 and z.shape[1] >= ff
+    y = torch.empty((z.shape[0], ff), dtype=z.dtype, device=z.device)
+    _hip.call("swl_relu_sq", _hip.ptr(y), _hip.ptr(z), z.shape[0], ff, z.stride(0), _hip.dtype_code3(z.dtype), _hip.stream())
+    return y
+
+
+def moe_experts_relu2(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, up: torch.Tensor,
+                      down: torch.Tensor) -> torch.Tensor:
+    """-> [T, width]: sum_j wts[t, j] * down[e_j] relu(up[e_j] h[t])^2 for experts without a gate. up [experts, ff, width],
+    down [experts, width, ff]. Large steps: assignments sorted by expert, a library product per expert; decode-sized 16-bit
+    steps: the expert-stationary matrix-core kernel; otherwise the per-assignment kernels."""
+    n, width = h.shape
+    experts, ff, _ = up.shape
+    top_k = idx.shape[1]
+    assert up.is_contiguous() and down.is_contiguous() and down.shape == (experts, width, ff)
+    assert up.dtype == down.dtype == h.dtype and idx.dtype == torch.int32 and wts.dtype == torch.float32
+    code, stream = _hip.dtype_code3(h.dtype), _hip.stream()
+    out = torch.empty((n, width), dtype=h.dtype, device=h.device)
+    if n * top_k >= GROUPED_MIN_ROWS_PER_EXPERT * experts and not torch.cuda.is_current_stream_capturing():
+        flat = idx.reshape(-1).long()
+        order = torch.argsort(flat, stable=True)
+        counts = torch.bincount(flat, minlength=experts).tolist()
+        where = torch.empty_like(order)
+        where[order] = torch.arange(order.numel(), device=order.device)
+        xs = h.index_select(0, order // top_k)
+        z = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
+        off = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(xs[off:off + c], up[e].t(), out=z[off:off + c])
+                off += c
+        y = relu_squared(z, ff)
+        rows = torch.empty((n * top_k, width), dtype=h.dtype, device=h.device)
+        off = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(y[off:off + c], down[e].t(), out=rows[off:off + c])
+                off += c
+        _hip.call("swl_moe_combine", _hip.ptr(out), _hip.ptr(rows), _hip.ptr(where), _hip.ptr(wts), n, width, top_k, code,
+                  stream)
+        return out
+    y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
+    if h.dtype != torch.float32 and _hip.load().swl_moe_expert_stationary_supported(n, width, ff, top_k, code):
+        _hip.call("swl_moe_expert_stationary", _hip.ptr(y), _hip.ptr(h), _hip.ptr(up), _hip.ptr(idx), n, experts, width, ff,
+                  top_k, 2, 0.0, code, stream)
+        rows = torch.empty((n * top_k, width), dtype=h.dtype, device=h.device)
+        _hip.call("swl_moe_expert_stationary", _hip.ptr(rows), _hip.ptr(y), _hip.ptr(down), _hip.ptr(idx), n, experts,
+                  width, ff, top_k, 0, 0.0, code, stream)
+        _hip.call("swl_moe_combine", _hip.ptr(out), _hip.ptr(rows), _hip.ptr(_identity(n * top_k, h.device)),
+                  _hip.ptr(wts), n, width, top_k, code, stream)
+        return out
+    _hip.call("swl_moe_up_relu2", _hip.ptr(y), _hip.ptr(h), _hip.ptr(up), _hip.ptr(idx), n, width, ff, top_k, code, stream)
+    _hip.call("swl_moe_down_combine", _hip.ptr(out), _hip.ptr(y), _hip.ptr(down), _hip.ptr(idx), _hip.ptr(wts), n, width,
+              ff, top_k, code, stream)
+    return out
+
+
 # From this many assignments per expert on (on average), a step's expert products are library GEMMs over the assignments
 # sorted by expert; below, every assignment streams its expert's rows (decode batches: capturable, no host read-back).
 GROUPED_MIN_ROWS_PER_EXPERT = 16
