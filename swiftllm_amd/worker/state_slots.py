@@ -103,5 +103,14 @@ class StateSlotManager:
             self._slot_of[sid] = slot
             self._parity[sid] = saved[1]
 
+    def snapshot(self, seq_ids: Sequence[int]):
+        """A copy of the slots of the given sequences (to undo a step that has to run twice)."""
+        rows = torch.tensor(sorted({self._slot_of[s] for s in seq_ids}), dtype=torch.long, device=self.pool.device)
+        return rows, self.pool.index_select(0, rows)
+
+    def restore(self, saved):
+        rows, data = saved
+        self.pool.index_copy_(0, rows, data)
+
     def live_sequences(self) -> List[int]:
         return sorted(self._slot_of)

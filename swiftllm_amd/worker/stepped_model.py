@@ -199,11 +199,16 @@ class SteppedModel:
             entry = None        # the metadata buffer was re-allocated: the capture points at the old one
         if entry is None:
             self.graph_captures += 1
-            warm = torch.cuda.Stream()      # one eager run first: nothing may be lazily initialised under capture
+            # one eager run first: nothing may be lazily initialised under capture. The replay below runs the step once more:
+            # writes into the block pool repeat themselves, recurrent state does not, so its slots are put back
+            saved = self.state.snapshot(plan.seq_ids_list) if self.state is not None else None
+            warm = torch.cuda.Stream()
             warm.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(warm):
                 self._logits(self._run_stack(dev, True), dev["want_rows"])
             torch.cuda.current_stream().wait_stream(warm)
+            if saved is not None:
+                self.state.restore(saved)
             while len(self._decode_graphs) >= self._MAX_DECODE_GRAPHS:
                 self._decode_graphs.pop(next(iter(self._decode_graphs)))
             if self._graph_pool is None:

@@ -54,23 +54,29 @@ def delta_scan(q, k, v, beta, g, state=None):
     return o, S
 
 
-def delta_mixer(h, W, pre, mx, eps):
-    n = h.shape[0]
+def delta_from_projections(qp, kp, vp, gp, bp, ap, W, pre, mx, eps):
+    """Raw projections (q, k [n, G * d], v, gate [n, H * e], b, a [n, H]) -> the mixer's output before W_o, [n, H * e]."""
+    n = qp.shape[0]
     H, G, d, e = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
-    q = silu(causal_conv(h @ W[pre + "q"].T, W[pre + "q.conv"])).view(n, G, d)
-    k = silu(causal_conv(h @ W[pre + "k"].T, W[pre + "k.conv"])).view(n, G, d)
-    v = silu(causal_conv(h @ W[pre + "v"].T, W[pre + "v.conv"])).view(n, H, e)
+    q = silu(causal_conv(qp, W[pre + "q.conv"])).view(n, G, d)
+    k = silu(causal_conv(kp, W[pre + "k.conv"])).view(n, G, d)
+    v = silu(causal_conv(vp, W[pre + "v.conv"])).view(n, H, e)
     q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * d ** -0.5
     k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
-    beta = torch.sigmoid(h @ W[pre + "b"].T)                                            # [n, H]
-    decay = torch.exp(-torch.exp(W[pre + "A_log"]) * torch.nn.functional.softplus(h @ W[pre + "a"].T + W[pre + "dt_bias"]))
-    gate = silu(h @ W[pre + "g"].T).view(n, H, e)
+    beta = torch.sigmoid(bp)
+    decay = torch.exp(-torch.exp(W[pre + "A_log"]) * torch.nn.functional.softplus(ap + W[pre + "dt_bias"]))
+    gate = silu(gp).view(n, H, e)
     out = torch.zeros(n, H, e, dtype=F64)
     for hd in range(H):
         kv = hd // (H // G)
         o, _ = delta_scan(q[:, kv], k[:, kv], v[:, hd], beta[:, hd], decay[:, hd])
         out[:, hd] = unit_rms(o, eps) * W[pre + "norm"] * gate[:, hd]
-    return out.reshape(n, H * e) @ W[pre + "o"].T
+    return out.reshape(n, H * e)
+
+
+def delta_mixer(h, W, pre, mx, eps):
+    parts = [h @ W[pre + name].T for name in ("q", "k", "v", "g", "b", "a")]
+    return delta_from_projections(*parts, W, pre, mx, eps) @ W[pre + "o"].T
 
 
 # ---- attention with a learned distance bias -------------------------------------------------------------------------------
@@ -96,21 +102,14 @@ def attention_keys_values(h, W, pre, mx, eps):
     return k.view(n, G, d), v.view(n, G, e)
 
 
-def attention_mixer(h, W, pre, mx, eps, kv=None):
-    """kv: (keys, values) of the layer this one borrows from, or None: its own."""
-    n = h.shape[0]
-    H, G, d, e = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
-    q = unit_rms(h @ W[pre + "q"].T, eps) * W[pre + "q.norm"]
-    temp = mx.get("q_temp")
-    if temp:
-        q = q * query_temperature(n, temp["coef"], temp["every"]).unsqueeze(1)
-    q = q.view(n, H, d)
-    k, v = attention_keys_values(h, W, pre, mx, eps) if kv is None else kv
+def attention_output(q, k, v, mx, rel=None):
+    """q [n, H, d] (normed, with its temperature), k [n, G, d], v [n, G, e], rel [rows, H] or None -> [n, H * e]: softmax over
+    every key j <= i of q_i . k_j * scale + rel[bucket(i - j)]."""
+    n, H, G = q.shape[0], mx["heads"], mx["kv_heads"]
     k = k.repeat_interleave(H // G, dim=1)
     v = v.repeat_interleave(H // G, dim=1)
     s = torch.einsum("ihd,jhd->hij", q, k) * mx["scale"]
-    if pre + "rel" in W:
-        rel = W[pre + "rel"]                  # [rows, H]
+    if rel is not None:
         row_of = torch.tensor([distance_bucket(dist, rel.shape[0], mx["bias_max"]) for dist in range(n)])
         dist = (torch.arange(n).unsqueeze(1) - torch.arange(n).unsqueeze(0)).clamp(min=0)
         s = s + rel[row_of[dist]].permute(2, 0, 1)
@@ -118,8 +117,23 @@ def attention_mixer(h, W, pre, mx, eps, kv=None):
     j = torch.arange(n).unsqueeze(0)
     s = s.masked_fill(j > i, float("-inf"))
     p = torch.softmax(s, dim=-1)
-    o = torch.einsum("hij,jhd->ihd", p, v).reshape(n, H * e)
-    return o @ W[pre + "o"].T
+    return torch.einsum("hij,jhd->ihd", p, v).reshape(n, -1)
+
+
+def normed_queries(qp, qn, mx, eps):
+    """qp [n, H * d] raw projection -> [n, H, d]: one RMS norm over the whole projection, then the temperature."""
+    q = unit_rms(qp, eps) * qn
+    temp = mx.get("q_temp")
+    if temp:
+        q = q * query_temperature(qp.shape[0], temp["coef"], temp["every"]).unsqueeze(1)
+    return q.view(qp.shape[0], mx["heads"], mx["dim"])
+
+
+def attention_mixer(h, W, pre, mx, eps, kv=None):
+    """kv: (keys, values) of the layer this one borrows from, or None: its own."""
+    q = normed_queries(h @ W[pre + "q"].T, W[pre + "q.norm"], mx, eps)
+    k, v = attention_keys_values(h, W, pre, mx, eps) if kv is None else kv
+    return attention_output(q, k, v, mx, W.get(pre + "rel")) @ W[pre + "o"].T
 
 
 # ---- feed-forwards ----------------------------------------------------------------------------------------------------------
@@ -186,3 +200,99 @@ def forward(cfg, W, tokens, taps=None):
         streams.append(x.clone())
     logits = norm_one_plus(x, W["final.norm"], eps) @ W["head"].T
     return logits, streams
+
+
+# ---- small configurations and random weights for the tests ----------------------------------------------------------------
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, scale=0.3, bias_max=40, temp=(0.4, 8), kv_from=None, mlp=None):
+    mixer = {"dim": dim, "heads": heads, "kv_heads": kv_heads, "scale": scale, "vdim": vdim}
+    if bias_max:
+        mixer["bias_max"] = bias_max
+    if temp:
+        mixer["q_temp"] = {"coef": temp[0], "every": temp[1]}
+    if kv_from is not None:
+        mixer["kv_from"] = kv_from
+    return {"type": "attention", "mixer": mixer, "mlp": mlp}
+
+
+def delta_layer(heads=4, kv_heads=2, dim=16, vdim=16, conv=4, mlp=None):
+    return {"type": "delta", "mixer": {"conv": conv, "dim": dim, "heads": heads, "kv_heads": kv_heads, "vdim": vdim},
+            "mlp": mlp}
+
+
+def dense_mlp(ff, limit=1.5):
+    return {"kind": "dense", "ff": ff, "limit": limit}
+
+
+def moe_mlp(ff, experts, top, scale=2.0, shared=None):
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "scale": scale}}
+    if shared:
+        mlp["shared"] = {"ff": shared}
+    return mlp
+
+
+def make_config(width=48, vocab=96, layers=None, taps=3, max_positions=256, eps=1e-5):
+    if layers is None:
+        layers = [attention_layer(mlp=dense_mlp(80)), delta_layer(mlp=moe_mlp(32, 6, 2, shared=40)),
+                  attention_layer(kv_from=0, mlp=moe_mlp(32, 4, 1))]
+    return {"architecture": "Lorulix", "canon": {"taps": taps}, "layers": layers, "max_positions": max_positions,
+            "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
+def make_weights(cfg, seed=0, bias_rows=12):
+    """Random bfloat16-representable weights with the checkpoint's names; sizes chosen so that every mechanism matters
+    (gates away from saturation, decays neither 0 nor 1, a distance bias of the size of the scores)."""
+    g = torch.Generator().manual_seed(seed)
+    w = cfg["width"]
+    taps = cfg["canon"]["taps"]
+
+    def rnd(*shape, s=1.0):
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
+
+    W = {"embed": rnd(cfg["vocab"], w), "pos": rnd(cfg["max_positions"], w, s=0.5), "final.norm": rnd(w, s=0.1),
+         "head": rnd(cfg["vocab"], w, s=w ** -0.5)}
+    for i, layer in enumerate(cfg["layers"]):
+        p, mx, mlp = f"l{i}.", layer["mixer"], layer.get("mlp")
+        for k in ("1", "2") if mlp else ("1",):
+            W[p + "norm" + k] = rnd(w, s=0.1)
+            W[p + "norm" + k + "b"] = rnd(w, s=0.1)
+            W[p + "canon" + k] = rnd(w, taps, s=0.4)
+            W[p + "rg" + k] = rnd(w, w, s=w ** -0.5)
+            W[p + "rg" + k + ".b"] = rnd(w, s=0.5)
+        H, G, d, e = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+        if layer["type"] == "attention":
+            W[p + "mix.q"] = rnd(H * d, w, s=w ** -0.5)
+            W[p + "mix.q.norm"] = (1.0 + 0.2 * torch.randn(H * d, generator=g)).to(torch.bfloat16)
+            if mx.get("kv_from") is None:
+                W[p + "mix.k"] = rnd(G * d, w, s=w ** -0.5)
+                W[p + "mix.v"] = rnd(G * e, w, s=w ** -0.5)
+                W[p + "mix.k.norm"] = (1.0 + 0.2 * torch.randn(G * d, generator=g)).to(torch.bfloat16)
+            if mx.get("bias_max"):
+                W[p + "mix.rel"] = rnd(bias_rows, H, s=1.5)
+            W[p + "mix.o"] = rnd(w, H * e, s=(H * e) ** -0.5)
+        else:
+            c = mx["conv"]
+            W[p + "mix.q"], W[p + "mix.q.conv"] = rnd(G * d, w, s=w ** -0.5), rnd(G * d, c, s=0.6)
+            W[p + "mix.k"], W[p + "mix.k.conv"] = rnd(G * d, w, s=w ** -0.5), rnd(G * d, c, s=0.6)
+            W[p + "mix.v"], W[p + "mix.v.conv"] = rnd(H * e, w, s=w ** -0.5), rnd(H * e, c, s=0.6)
+            W[p + "mix.b"], W[p + "mix.a"] = rnd(H, w, s=w ** -0.5), rnd(H, w, s=w ** -0.5)
+            W[p + "mix.A_log"], W[p + "mix.dt_bias"] = rnd(H, s=0.5), rnd(H, s=0.5)
+            W[p + "mix.norm"] = (1.0 + 0.2 * torch.randn(e, generator=g)).to(torch.bfloat16)
+            W[p + "mix.g"] = rnd(H * e, w, s=w ** -0.5)
+            W[p + "mix.o"] = rnd(w, H * e, s=(H * e) ** -0.5)
+        if not mlp:
+            continue
+        if mlp["kind"] == "dense":
+            ff = mlp["ff"]
+            W[p + "mlp.gate"], W[p + "mlp.up"] = rnd(ff, w, s=2 * w ** -0.5), rnd(ff, w, s=2 * w ** -0.5)
+            W[p + "mlp.down"] = rnd(w, ff, s=ff ** -0.5)
+        else:
+            ff = mlp["expert"]["ff"]
+            W[p + "mlp.router"] = rnd(mlp["router"]["experts"], w, s=2 * w ** -0.5)
+            for x in range(mlp["router"]["experts"]):
+                W[f"{p}mlp.e{x}.up"] = rnd(ff, w, s=w ** -0.5)
+                W[f"{p}mlp.e{x}.down"] = rnd(w, ff, s=ff ** -0.5)
+            if mlp.get("shared"):
+                fs = mlp["shared"]["ff"]
+                W[p + "mlp.shared.up"], W[p + "mlp.shared.down"] = rnd(fs, w, s=w ** -0.5), rnd(w, fs, s=fs ** -0.5)
+                W[p + "mlp.shared.sg"] = rnd(1, w, s=w ** -0.5)
+    return W
