@@ -95,8 +95,9 @@ def parse_args():
                     help="top: filler sequences occupy the low block ids, the run's sequences get the highest ones")
     ap.add_argument("--no-reference", action="store_true", help="skip the reference-Triton child run")
     ap.add_argument("--compare-designs", action="store_true",
-                    help="instead of the headline workload: prefill and decode throughput of Kekapel beside LLaMA at equal "
-                         "layer sizes (random weights), one JSON line with both")
+                    help="instead of the headline workload: prefill and decode throughput of the other designs (Kekapel, "
+                         "Lorulix) beside LLaMA at equal layer sizes (random weights), one JSON line with all")
+    ap.add_argument("--compare", default="llama,kekapel,lorulix", help="designs that --compare-designs runs (comma list)")
     ap.add_argument("--compare-sizes", default="small,medium", help="comma list out of " + ",".join(COMPARE_SIZES))
     return ap.parse_args()
 
@@ -123,7 +124,24 @@ def _compare_configs(sz, positions):
     layers = [dict(type="attention", mixer=mixer, mlp=(moe if i % 2 else dense)) for i in range(sz["layers"])]
     kekapel = dict(architecture="Kekapel", embedding=dict(scale=1.0), layers=layers, max_positions=positions,
                    norm=dict(eps=1e-6), residual_mult=0.5, vocab=sz["vocab"], width=sz["width"])
-    return llama, kekapel
+    # Lorulix at the same sizes: attention with keys of its own / delta rule / attention on the first one's keys, in turn;
+    # the same dense and expert widths as Kekapel (plus a shared expert of an expert's width), convolutions of 3 and 4 taps
+    attn = dict(dim=sz["dim"], vdim=sz["dim"], heads=sz["heads"], kv_heads=sz["kv_heads"], scale=sz["dim"] ** -0.5,
+                bias_max=1024, q_temp=dict(coef=0.1, every=256))
+    delta = dict(dim=sz["dim"], vdim=sz["dim"], heads=sz["heads"], kv_heads=sz["kv_heads"], conv=4)
+    lmoe = dict(kind="moe", expert=dict(ff=sz["ff"] // 4), router=dict(experts=8, top=2, scale=1.0),
+                shared=dict(ff=sz["ff"] // 4))
+    ldense = dict(kind="dense", ff=sz["ff"], limit=7.0)
+    llayers = []
+    for i in range(sz["layers"]):
+        kind = i % 3
+        mixer = dict(attn) if kind != 1 else dict(delta)
+        if kind == 2:
+            mixer["kv_from"] = i - 2
+        llayers.append(dict(type="delta" if kind == 1 else "attention", mixer=mixer, mlp=(lmoe if i % 2 else ldense)))
+    lorulix = dict(architecture="Lorulix", canon=dict(taps=3), layers=llayers, max_positions=positions,
+                   norm=dict(eps=1e-6), vocab=sz["vocab"], width=sz["width"])
+    return llama, kekapel, lorulix
 
 
 def _compare_one(cfg, dtype, prompt_len, prompt_batch, decode_batch, decode_ctx, steps, warmup):
@@ -184,19 +202,23 @@ def _compare_one(cfg, dtype, prompt_len, prompt_batch, decode_batch, decode_ctx,
 
 
 def run_compare_designs(args):
-    """Both designs at every requested size -> one JSON-able dict (rates in tokens/s; ratio = Kekapel / LLaMA)."""
+    """The designs at every requested size -> one JSON-able dict (rates in tokens/s; ratios: Kekapel / LLaMA, Lorulix /
+    Kekapel — the closest existing design: the same worker, stream and expert kernels — and Lorulix / LLaMA)."""
     results = {}
     for name in [s for s in args.compare_sizes.split(",") if s]:
         sz = COMPARE_SIZES[name]
         prompt_len, prompt_batch, decode_batch, decode_ctx = 2048, 4, 32, 1024
-        llama, kekapel = _compare_configs(sz, prompt_len + 256)
+        configs = dict(zip(("llama", "kekapel", "lorulix"), _compare_configs(sz, prompt_len + 256)))
         rec = {"sizes": sz, "prompt": [prompt_batch, prompt_len], "decode": [decode_batch, decode_ctx]}
-        for label, cfg in (("llama", llama), ("kekapel", kekapel)):
-            rec[label] = _compare_one(cfg, args.dtype, prompt_len, prompt_batch, decode_batch, decode_ctx,
+        for label in [d for d in args.compare.split(",") if d]:
+            rec[label] = _compare_one(configs[label], args.dtype, prompt_len, prompt_batch, decode_batch, decode_ctx,
                                       min(args.steps, 32), min(args.warmup, 8))
             print(f"[compare] {name} {label}: {rec[label]}", file=sys.stderr, flush=True)
-        rec["prefill_ratio"] = rec["kekapel"]["prefill_tokens_per_s"] / rec["llama"]["prefill_tokens_per_s"]
-        rec["decode_ratio"] = rec["kekapel"]["decode_tokens_per_s"] / rec["llama"]["decode_tokens_per_s"]
+        for a, b, key in (("kekapel", "llama", ""), ("lorulix", "kekapel", "lorulix_vs_kekapel_"),
+                          ("lorulix", "llama", "lorulix_vs_llama_")):
+            if a in rec and b in rec:
+                rec[key + "prefill_ratio"] = rec[a]["prefill_tokens_per_s"] / rec[b]["prefill_tokens_per_s"]
+                rec[key + "decode_ratio"] = rec[a]["decode_tokens_per_s"] / rec[b]["decode_tokens_per_s"]
         results[name] = rec
     return {"metric": "design_comparison_tokens_per_s", "dtype": args.dtype, "data": "synthetic", "n_gpus": 1,
             "results": results}
