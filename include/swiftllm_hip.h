@@ -609,16 +609,17 @@ int swl_causal_conv_state(void *out, int64_t out_stride, const void *h, int64_t 
                           int32_t taps, int32_t add_input, int32_t dtype, swl_stream_t stream);
 
 /* ---- gated delta rule (csrc/delta_rule.hip) --------------------------------------------------------------------------------
- * swl_delta_prep: proj rows [q | k | v | gate | b | a] -> qn, kn [T, qk heads * dim], vv [T, heads * vdim], beta, decay
+ * swl_delta_prep: proj rows [q | k | v | gate | b | a] -> qn, kn [T, qk heads * dim], kq [T, qk heads] (their dot
+ * products), vv [T, heads * vdim], beta, decay
  * [T, heads], all fp32 (convolution + SiLU, unit norms, sigmoid, exp(-exp(A_log) softplus(a + dt_bias))).
  * swl_delta_rule: o[T, heads * vdim] (fp32) and the states [heads, dim, vdim] at s_off inside the slots, one portion per
  * (seq_row0, seq_cnt) entry. swl_gated_head_rmsnorm: out = o / rms(o over vdim) * w[vdim] * silu(gate). */
-int swl_delta_prep(float *qn, float *kn, float *vv, float *beta, float *decay, const void *proj, int64_t proj_stride,
+int swl_delta_prep(float *qn, float *kn, float *kq, float *vv, float *beta, float *decay, const void *proj, int64_t proj_stride,
                    const float *conv_w, const float *a_log, const float *dt_bias, float *state, int64_t slot_stride,
                    int64_t tail_off, const int32_t *tok_pos, const int32_t *tok_start, const int32_t *tok_state,
                    const int32_t *tok_seq, int64_t num_tokens, int32_t num_heads, int32_t num_qk_heads, int32_t dim,
                    int32_t vdim, int32_t taps, int32_t dtype, swl_stream_t stream);
-int swl_delta_rule(float *o, const float *qn, const float *kn, const float *vv, const float *beta, const float *decay,
+int swl_delta_rule(float *o, const float *qn, const float *kn, const float *kq, const float *vv, const float *beta, const float *decay,
                    float *state, int64_t slot_stride, int64_t s_off, const int32_t *seq_row0, const int32_t *seq_cnt,
                    const int32_t *tok_pos, const int32_t *tok_state, int32_t num_seqs, int32_t num_heads,
                    int32_t num_qk_heads, int32_t dim, int32_t vdim, swl_stream_t stream);

@@ -116,9 +116,9 @@ SIGNATURES = {
                                  _F32, _I32, _I32, _P],
     "swl_gated_add_rmsnorm": [_P, _P, _P, _P, _I64, _P, _I64, _P, _P, _P, _P, _P, _F32, _I64, _I32, _I32, _P],
     "swl_causal_conv_state": [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
-    "swl_delta_prep": [_P, _P, _P, _P, _P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32,
+    "swl_delta_prep": [_P, _P, _P, _P, _P, _P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32,
                        _I32, _I32, _I32, _P],
-    "swl_delta_rule": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
+    "swl_delta_rule": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
     "swl_gated_head_rmsnorm": [_P, _P, _P, _I64, _P, _F32, _I64, _I32, _I32, _I32, _P],
 }
 # Entry points that do not follow the "int rc = f(...)" convention.

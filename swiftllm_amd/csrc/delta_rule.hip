@@ -9,9 +9,10 @@
 //                    beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias)); everything after the loads is fp32.
 //   swl_delta_rule:  one workgroup per (portion, head). The columns of S are independent recurrences, so a column belongs
 //                    to L adjacent lanes, each holding dim / L of its elements in registers; per token the lanes exchange
-//                    three partial dot products (S^T k, S^T q, k . q) through DPP and o = S^T q + u (k . q) needs no second
+//                    two partial dot products (S^T k, S^T q) through DPP and o = S^T q + u (k . q, from the prep) needs no second
 //                    pass over the state. q, k, v, beta, g of 16 tokens at a time are staged in LDS. The token loop is
-//                    sequential whatever the cut of the sequence into steps: the same operations in the same order.
+//                    sequential whatever the cut of the sequence into steps: the same operations in the same order. When
+//                    a step has few (portion, head) pairs the columns of a head are shared out over several workgroups.
 //   swl_gated_head_rmsnorm: out = o / rms(o over vdim) * w * silu(gate), per head.
 #include "swl_common.h"
 #include "conv_tail.h"
@@ -25,8 +26,8 @@ __device__ __forceinline__ float dr_sigmoid(float z) { return 1.0f / (1.0f + exp
 
 template <typename T>
 __global__ __launch_bounds__(kDpThreads) void delta_prep_kernel(
-    float *qn, float *kn, float *vv, float *beta, float *decay, const T *proj, int64_t proj_stride, const float *conv_w,
-    const float *a_log, const float *dt_bias, float *state, int64_t slot_stride, int64_t tail_off, const int32_t *tok_pos,
+    float *qn, float *kn, float *kq, float *vv, float *beta, float *decay, const T *proj, int64_t proj_stride,
+    const float *conv_w, const float *a_log, const float *dt_bias, float *state, int64_t slot_stride, int64_t tail_off, const int32_t *tok_pos,
     const int32_t *tok_start, const int32_t *tok_state, const int32_t *tok_seq, int64_t num_tokens, int H, int G, int d,
     int dv, int taps) {
     extern __shared__ float act[];      // [2 G d + H dv] convolved, activated channels
@@ -43,19 +44,24 @@ __global__ __launch_bounds__(kDpThreads) void delta_prep_kernel(
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const float qscale = 1.0f / sqrtf(static_cast<float>(d));
-    for (int hh = wave; hh < 2 * G; hh += kDpThreads / 64) {
-        const float *src = act + hh * d;
-        float ss = 0.f;
-        for (int e = lane; e < d; e += 64) ss += src[e] * src[e];
-        ss = wave_allreduce_sum(ss);
-        const float r = 1.0f / sqrtf(ss + 1e-6f);
-        if (hh < G) {
-            float *dst = qn + t * qk + hh * d;
-            for (int e = lane; e < d; e += 64) dst[e] = src[e] * r * qscale;
-        } else {
-            float *dst = kn + t * qk + (hh - G) * d;
-            for (int e = lane; e < d; e += 64) dst[e] = src[e] * r;
+    for (int g = wave; g < G; g += kDpThreads / 64) {       // q head g and k head g: unit norms and their dot product
+        const float *qsrc = act + g * d, *ksrc = act + qk + g * d;
+        float sq = 0.f, sk = 0.f, dot = 0.f;
+        for (int e = lane; e < d; e += 64) {
+            sq += qsrc[e] * qsrc[e];
+            sk += ksrc[e] * ksrc[e];
+            dot += qsrc[e] * ksrc[e];
         }
+        sq = wave_allreduce_sum(sq);
+        sk = wave_allreduce_sum(sk);
+        dot = wave_allreduce_sum(dot);
+        const float rq = qscale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+        float *qdst = qn + t * qk + g * d, *kdst = kn + t * qk + g * d;
+        for (int e = lane; e < d; e += 64) {
+            qdst[e] = qsrc[e] * rq;
+            kdst[e] = ksrc[e] * rk;
+        }
+        if (lane == 0) kq[t * G + g] = dot * rq * rk;
     }
     for (int i = threadIdx.x; i < H * dv; i += kDpThreads) vv[t * H * dv + i] = act[2 * qk + i];
     for (int h = threadIdx.x; h < H; h += kDpThreads) {
@@ -72,67 +78,99 @@ __device__ __forceinline__ float dr_group_sum(float v) {
     return group_allreduce_sum<L>(v);
 }
 
-template <int MAXDS, int L>
-__global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float *qn, const float *kn, const float *vv,
+// LDS rows of q and k are padded by 4 floats per lane slice: the L lanes of a column read L different 16-byte pieces at
+// once, and without the padding slices of 8 / 16 / 32 floats start in the same banks.
+__host__ __device__ inline int dr_row_floats(int d, int L) { return d + 4 * L; }
+
+template <int MAXDS, int L, bool EXACT>
+__global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float *qn, const float *kn, const float *kqn,
+                                                          const float *vv,
                                                           const float *beta, const float *decay, float *state,
                                                           int64_t slot_stride, int64_t s_off, const int32_t *seq_row0,
                                                           const int32_t *seq_cnt, const int32_t *tok_pos,
-                                                          const int32_t *tok_state, int H, int G, int d, int dv) {
+                                                          const int32_t *tok_state, int H, int G, int d, int dv, int cpw) {
     extern __shared__ float lds[];
-    float *qs = lds;                        // [chunk][d]
-    float *ks = qs + kDrChunk * d;          // [chunk][d]
-    float *vs = ks + kDrChunk * d;          // [chunk][dv]
-    float *bs = vs + kDrChunk * dv;         // [chunk]
+    const int dp = dr_row_floats(d, L);
+    float *qs = lds;                        // [chunk][dp]
+    float *ks = qs + kDrChunk * dp;         // [chunk][dp]
+    float *vs = ks + kDrChunk * dp;         // [chunk][cpw]
+    float *bs = vs + kDrChunk * cpw;        // [chunk]
     float *gs = bs + kDrChunk;              // [chunk]
+    float *kqs = gs + kDrChunk;             // [chunk] k . q of the token's (normed) q / k head
     const int seq = blockIdx.x, h = blockIdx.y;
+    const int col0 = blockIdx.z * cpw;      // this workgroup's columns of the state (independent recurrences)
     const int row0 = seq_row0[seq], cnt = seq_cnt[seq];
     const int kvh = h / (H / G);
-    const int col = threadIdx.x / L, l = threadIdx.x % L;
-    const int ds = d / L, i0 = l * ds;
+    const int lc = threadIdx.x / L, l = threadIdx.x % L;
+    const int col = col0 + lc;
+    const int ds = EXACT ? MAXDS : d / L, i0 = l * ds;      // (EXACT: the slice fills the register array, no predicates)
     float *S = state + static_cast<int64_t>(tok_state[row0] >> 1) * slot_stride + s_off + static_cast<int64_t>(h) * d * dv;
     float s[MAXDS];
     const bool fresh = tok_pos[row0] == 0;      // a sequence starts from the zero state whatever the slot held
 #pragma unroll
     for (int i = 0; i < MAXDS; ++i) s[i] = (i < ds && !fresh) ? S[static_cast<int64_t>(i0 + i) * dv + col] : 0.f;
     const int qk = G * d, hv = H * dv;
+    const bool quads = EXACT || (ds & 3) == 0;  // 16-byte LDS reads
     for (int c0 = 0; c0 < cnt; c0 += kDrChunk) {
         const int cn = min(kDrChunk, cnt - c0);
         __syncthreads();        // the previous chunk has been consumed
         for (int i = threadIdx.x; i < cn * d; i += blockDim.x) {
             const int j = i / d, e = i - j * d;
             const int64_t r = row0 + c0 + j;
-            qs[i] = qn[r * qk + kvh * d + e];
-            ks[i] = kn[r * qk + kvh * d + e];
+            const int at = j * dp + e + 4 * (e / ds);
+            qs[at] = qn[r * qk + kvh * d + e];
+            ks[at] = kn[r * qk + kvh * d + e];
         }
-        for (int i = threadIdx.x; i < cn * dv; i += blockDim.x) {
-            const int j = i / dv, e = i - j * dv;
-            vs[i] = vv[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + e];
+        for (int i = threadIdx.x; i < cn * cpw; i += blockDim.x) {
+            const int j = i / cpw, e = i - j * cpw;
+            vs[i] = vv[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + col0 + e];
         }
         for (int j = threadIdx.x; j < cn; j += blockDim.x) {
             bs[j] = beta[static_cast<int64_t>(row0 + c0 + j) * H + h];
             gs[j] = decay[static_cast<int64_t>(row0 + c0 + j) * H + h];
+            kqs[j] = kqn[static_cast<int64_t>(row0 + c0 + j) * G + kvh];
         }
         __syncthreads();
+#pragma unroll 2
         for (int j = 0; j < cn; ++j) {
-            const float g = gs[j], b = bs[j];
-            const float *kj = ks + j * d + i0, *qj = qs + j * d + i0;
-            float sk = 0.f, sq = 0.f, kq = 0.f;
+            const float g = gs[j], b = bs[j], kq = kqs[j];
+            const float *kj = ks + j * dp + l * (ds + 4), *qj = qs + j * dp + l * (ds + 4);
+            float kr[MAXDS], qr[MAXDS];
+            if (quads) {
+#pragma unroll
+                for (int i = 0; i < MAXDS; i += 4) {
+                    if (EXACT || i < ds) {
+                        const float4_t k4 = *reinterpret_cast<const float4_t *>(kj + i);
+                        const float4_t q4 = *reinterpret_cast<const float4_t *>(qj + i);
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            kr[i + c] = k4[c];
+                            qr[i + c] = q4[c];
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < MAXDS; ++i) {
+                    kr[i] = i < ds ? kj[i] : 0.f;
+                    qr[i] = i < ds ? qj[i] : 0.f;
+                }
+            }
+            float sk = 0.f, sq = 0.f;
 #pragma unroll
             for (int i = 0; i < MAXDS; ++i) {
-                if (i < ds) {
+                if (EXACT || i < ds) {
                     s[i] *= g;
-                    sk += s[i] * kj[i];
-                    sq += s[i] * qj[i];
-                    kq += kj[i] * qj[i];
+                    sk += s[i] * kr[i];
+                    sq += s[i] * qr[i];
                 }
             }
             sk = dr_group_sum<L>(sk);
             sq = dr_group_sum<L>(sq);
-            kq = dr_group_sum<L>(kq);
-            const float u = b * (vs[j * dv + col] - sk);
+            const float u = b * (vs[j * cpw + lc] - sk);
 #pragma unroll
             for (int i = 0; i < MAXDS; ++i)
-                if (i < ds) s[i] += kj[i] * u;
+                if (EXACT || i < ds) s[i] += kr[i] * u;
             if (l == 0) o[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + col] = sq + u * kq;
         }
     }
@@ -169,25 +207,29 @@ inline int dr_lanes(int d, int dv) {
 
 template <int L>
 int launch_dr(int ds, dim3 grid, dim3 block, size_t lds, hipStream_t s, float *o, const float *qn, const float *kn,
-              const float *vv, const float *beta, const float *decay, float *state, int64_t slot_stride, int64_t s_off,
+              const float *kq, const float *vv, const float *beta, const float *decay, float *state, int64_t slot_stride, int64_t s_off,
               const int32_t *seq_row0, const int32_t *seq_cnt, const int32_t *tok_pos, const int32_t *tok_state, int H,
-              int G, int d, int dv) {
-#define SWL_DR_LAUNCH(M)                                                                                                     \
-    hipLaunchKernelGGL((delta_rule_kernel<M, L>), grid, block, lds, s, o, qn, kn, vv, beta, decay, state, slot_stride, s_off, \
-                       seq_row0, seq_cnt, tok_pos, tok_state, H, G, d, dv)
-    if (ds <= 8) SWL_DR_LAUNCH(8);
-    else if (ds <= 16) SWL_DR_LAUNCH(16);
-    else if (ds <= 32) SWL_DR_LAUNCH(32);
-    else if (ds <= 64) SWL_DR_LAUNCH(64);
-    else if (ds <= 128) SWL_DR_LAUNCH(128);
+              int G, int d, int dv, int cpw) {
+#define SWL_DR_LAUNCH1(M, X)                                                                                                 \
+    hipLaunchKernelGGL((delta_rule_kernel<M, L, X>), grid, block, lds, s, o, qn, kn, kq, vv, beta, decay, state, slot_stride, \
+                       s_off, seq_row0, seq_cnt, tok_pos, tok_state, H, G, d, dv, cpw)
+#define SWL_DR_LAUNCH(M)                   \
+    if (ds == M) SWL_DR_LAUNCH1(M, true);  \
+    else SWL_DR_LAUNCH1(M, false)
+    if (ds <= 8) { SWL_DR_LAUNCH(8); }
+    else if (ds <= 16) { SWL_DR_LAUNCH(16); }
+    else if (ds <= 32) { SWL_DR_LAUNCH(32); }
+    else if (ds <= 64) { SWL_DR_LAUNCH(64); }
+    else if (ds <= 128) { SWL_DR_LAUNCH(128); }
     else return SWL_ERR_UNSUPPORTED;
 #undef SWL_DR_LAUNCH
+#undef SWL_DR_LAUNCH1
     return check_launch();
 }
 
 } // namespace swl
 
-extern "C" int swl_delta_prep(float *qn, float *kn, float *vv, float *beta, float *decay, const void *proj,
+extern "C" int swl_delta_prep(float *qn, float *kn, float *kq, float *vv, float *beta, float *decay, const void *proj,
                               int64_t proj_stride, const float *conv_w, const float *a_log, const float *dt_bias,
                               float *state, int64_t slot_stride, int64_t tail_off, const int32_t *tok_pos,
                               const int32_t *tok_start, const int32_t *tok_state, const int32_t *tok_seq,
@@ -198,21 +240,22 @@ extern "C" int swl_delta_prep(float *qn, float *kn, float *vv, float *beta, floa
     const int64_t C = 2LL * num_qk_heads * dim + static_cast<int64_t>(num_heads) * vdim;
     if (proj_stride < C + static_cast<int64_t>(num_heads) * vdim + 2 * num_heads) return SWL_ERR_BAD_ARG;
     if (num_tokens == 0) return SWL_OK;
-    if (!qn || !kn || !vv || !beta || !decay || !proj || !conv_w || !a_log || !dt_bias || !tok_pos || !tok_start || !tok_seq)
+    if (!qn || !kn || !kq || !vv || !beta || !decay || !proj || !conv_w || !a_log || !dt_bias || !tok_pos || !tok_start || !tok_seq)
         return SWL_ERR_BAD_ARG;
     if (taps > 1 && (!state || !tok_state)) return SWL_ERR_BAD_ARG;
     const size_t lds = static_cast<size_t>(C) * sizeof(float);
     if (num_tokens > 0x7fffffffLL || lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
     SWL_DISPATCH_DTYPE3(dtype, T, {
         hipLaunchKernelGGL((swl::delta_prep_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kDpThreads), lds,
-                           static_cast<hipStream_t>(stream), qn, kn, vv, beta, decay, static_cast<const T *>(proj),
+                           static_cast<hipStream_t>(stream), qn, kn, kq, vv, beta, decay, static_cast<const T *>(proj),
                            proj_stride, conv_w, a_log, dt_bias, state, slot_stride, tail_off, tok_pos, tok_start,
                            tok_state, tok_seq, num_tokens, num_heads, num_qk_heads, dim, vdim, taps);
     });
     return swl::check_launch();
 }
 
-extern "C" int swl_delta_rule(float *o, const float *qn, const float *kn, const float *vv, const float *beta,
+extern "C" int swl_delta_rule(float *o, const float *qn, const float *kn, const float *kq, const float *vv,
+                              const float *beta,
                               const float *decay, float *state, int64_t slot_stride, int64_t s_off,
                               const int32_t *seq_row0, const int32_t *seq_cnt, const int32_t *tok_pos,
                               const int32_t *tok_state, int32_t num_seqs, int32_t num_heads, int32_t num_qk_heads,
@@ -220,18 +263,23 @@ extern "C" int swl_delta_rule(float *o, const float *qn, const float *kn, const 
     if (num_seqs < 0 || num_heads <= 0 || num_qk_heads <= 0 || dim <= 0 || vdim <= 0 || num_heads % num_qk_heads)
         return SWL_ERR_BAD_ARG;
     if (num_seqs == 0) return SWL_OK;
-    if (!o || !qn || !kn || !vv || !beta || !decay || !state || !seq_row0 || !seq_cnt || !tok_pos || !tok_state)
+    if (!o || !qn || !kn || !kq || !vv || !beta || !decay || !state || !seq_row0 || !seq_cnt || !tok_pos || !tok_state)
         return SWL_ERR_BAD_ARG;
     if (vdim > 1024 || num_heads > 65535) return SWL_ERR_UNSUPPORTED;
     const int L = swl::dr_lanes(dim, vdim);
     const int ds = dim / L;
-    const size_t lds = (static_cast<size_t>(swl::kDrChunk) * (2 * dim + vdim + 2)) * sizeof(float);
+    // columns per workgroup: all of them when there are (portion, head) pairs enough to fill the chip (decode batches); a
+    // long prompt alone is a sequential walk, so its columns are shared out over more workgroups (down to 16 columns each)
+    int cpw = vdim;
+    while (static_cast<int64_t>(num_seqs) * num_heads * (vdim / cpw) < 512 && cpw % 2 == 0 && cpw > 16) cpw /= 2;
+    const size_t lds = (static_cast<size_t>(swl::kDrChunk) * (2 * swl::dr_row_floats(dim, L) + cpw + 3)) * sizeof(float);
     if (lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
-    const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads)), block(static_cast<unsigned>(vdim * L));
+    const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>(vdim / cpw));
+    const dim3 block(static_cast<unsigned>(cpw * L));
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define SWL_DR_L(LL)                                                                                                         \
-    case LL: return swl::launch_dr<LL>(ds, grid, block, lds, s, o, qn, kn, vv, beta, decay, state, slot_stride, s_off,       \
-                                       seq_row0, seq_cnt, tok_pos, tok_state, num_heads, num_qk_heads, dim, vdim)
+    case LL: return swl::launch_dr<LL>(ds, grid, block, lds, s, o, qn, kn, kq, vv, beta, decay, state, slot_stride, s_off,       \
+                                       seq_row0, seq_cnt, tok_pos, tok_state, num_heads, num_qk_heads, dim, vdim, cpw)
     switch (L) {
         SWL_DR_L(1);
         SWL_DR_L(2);

@@ -19,7 +19,7 @@ constexpr int kWmThreads = 256;
 constexpr int kWmWaves = 4;
 constexpr int kWmTile = 16;     // queries per tile = keys per page = MFMA edge
 
-template <typename T, int D, int DV, int HPW, int NW>
+template <typename T, int D, int DV, int HPW, int NW, bool MIX>
 __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk,
@@ -38,9 +38,12 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // (tells the compiler that it is wave-uniform)
     const int li = lane & 15, lq = lane >> 4;       // query (or operand row) index; quarter
-    // mixed scores come out in base-2 exponent units; without a matrix every head keeps its own scores
-    for (int i = tid; i < H * H; i += NW * 64) tk[i] = talk ? talk[i] * kLog2e : (i / H == i % H ? kLog2e : 0.f);
-    __syncthreads();
+    // mixed scores come out in base-2 exponent units. MIX = false (no matrix): every head keeps its own scores, which then
+    // never leave the registers of the wave that made them — no LDS, no barriers
+    if constexpr (MIX) {
+        for (int i = tid; i < H * H; i += NW * 64) tk[i] = talk[i] * kLog2e;
+        __syncthreads();
+    }
     const int p0 = __builtin_amdgcn_readfirstlane(tok_pos[row0]);
     const int32_t *bt = block_table + static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tok_seq[row0])) * max_blocks_per_seq;
     const int rep = H / G;
@@ -122,6 +125,11 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
             for (int hh = 0; hh < HPW; ++hh) fetch_v(hh);
         }
         // ---- 1. capped scores of this wave's heads -> LDS -------------------------------------------------------------------
+        float mixed[HPW][4];
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mixed[hh][r] = 0.f;
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int g = h0 + hh;
@@ -150,10 +158,15 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
                     else
                         st[r] *= scale;
                 }
-                *reinterpret_cast<float4_t *>(&s_lds[(g * 64 + lane) * 4]) = st;
+                if constexpr (MIX) {
+                    *reinterpret_cast<float4_t *>(&s_lds[(g * 64 + lane) * 4]) = st;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) mixed[hh][r] = st[r] * kLog2e;
+                }
             }
         }
-        __syncthreads();
+        if constexpr (MIX) __syncthreads();
         blk_next = __builtin_amdgcn_readfirstlane(nxt);
         if constexpr (PIPE) {
             if (kb < kb1) fetch_k(blk_next);
@@ -166,12 +179,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
             const int kp = kpos0 + r;
             ok[r] = qok && kp <= qpos && (window <= 0 || kp > qpos - window);
         }
-        float mixed[HPW][4];
-#pragma unroll
-        for (int hh = 0; hh < HPW; ++hh)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) mixed[hh][r] = 0.f;
-        for (int g = 0; g < H; ++g) {
+        for (int g = 0; MIX && g < H; ++g) {
             const float4_t sv = *reinterpret_cast<const float4_t *>(&s_lds[(g * 64 + lane) * 4]);
 #pragma unroll
             for (int hh = 0; hh < HPW; ++hh) {
@@ -230,7 +238,9 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
                 }
             }
         }
-        if (nbuf == 1) __syncthreads();     // every wave is done with this page's scores before the next page overwrites them
+        if constexpr (MIX) {
+            if (nbuf == 1) __syncthreads();     // every wave is done with this page's scores before the next page overwrites them
+        }
     }
     // ---- epilogue: O[query li][h][ct * 16 + 4 lq + r] = O^T / l -------------------------------------------------------------------
 #pragma unroll
@@ -295,9 +305,12 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
               const float *talk, const float *rel, int rel_len, int H, int G, int64_t qs, int window, float scale,
               float softcap, int mb, int64_t bs,
               float *po, float *pml, int64_t nt, int nbuf) {
-#define SWL_WM_LAUNCH(HPW, NW)                                                                                          \
-    hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW, NW>), grid, dim3(NW * 64), lds, s, out, q, kc, vc, bt, ts, \
-                       tp, r0, cn, talk, rel, rel_len, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf)
+#define SWL_WM_LAUNCH1(HPW, NW, MIX)                                                                                         \
+    hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW, NW, MIX>), grid, dim3(NW * 64), MIX ? lds : 0, s, out, q, kc, \
+                       vc, bt, ts, tp, r0, cn, talk, rel, rel_len, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf)
+#define SWL_WM_LAUNCH(HPW, NW)          \
+    if (talk) SWL_WM_LAUNCH1(HPW, NW, true); \
+    else SWL_WM_LAUNCH1(HPW, NW, false)
     // heads per wave x waves: up to 16 heads on four waves, more on eight (four heads per wave at most: the accumulators of
     // eight 128-wide heads do not fit a wave's registers)
     switch (hpw) {
@@ -308,6 +321,7 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
     default: return SWL_ERR_UNSUPPORTED;
     }
 #undef SWL_WM_LAUNCH
+#undef SWL_WM_LAUNCH1
     if (grid.y > 1) {
         const int64_t rows = nt * H;
         hipLaunchKernelGGL((window_attn_combine_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(DV < 256 ? 64 : 256), 0, s,

@@ -21,16 +21,17 @@ def delta_rule_mixer(proj: torch.Tensor, conv_w: torch.Tensor, a_log: torch.Tens
     dev, f32 = proj.device, torch.float32
     qn = torch.empty((n, G * d), dtype=f32, device=dev)
     kn = torch.empty((n, G * d), dtype=f32, device=dev)
+    kq = torch.empty((n, G), dtype=f32, device=dev)
     vv = torch.empty((n, H * dv), dtype=f32, device=dev)
     beta = torch.empty((n, H), dtype=f32, device=dev)
     decay = torch.empty((n, H), dtype=f32, device=dev)
     code, stream = _hip.dtype_code3(proj.dtype), _hip.stream()
-    _hip.call("swl_delta_prep", _hip.ptr(qn), _hip.ptr(kn), _hip.ptr(vv), _hip.ptr(beta), _hip.ptr(decay), _hip.ptr(proj),
+    _hip.call("swl_delta_prep", _hip.ptr(qn), _hip.ptr(kn), _hip.ptr(kq), _hip.ptr(vv), _hip.ptr(beta), _hip.ptr(decay), _hip.ptr(proj),
               proj.stride(0), _hip.ptr(conv_w), _hip.ptr(a_log), _hip.ptr(dt_bias), _hip.ptr(st.pool), st.pool.stride(0),
               int(tail_off), _hip.ptr(st.tok_pos), _hip.ptr(st.tok_start), _hip.ptr(st.tok_state), _hip.ptr(st.tok_seq), n,
               H, G, d, dv, mixer.conv_taps, code, stream)
     o = torch.empty((n, H * dv), dtype=f32, device=dev)
-    _hip.call("swl_delta_rule", _hip.ptr(o), _hip.ptr(qn), _hip.ptr(kn), _hip.ptr(vv), _hip.ptr(beta), _hip.ptr(decay),
+    _hip.call("swl_delta_rule", _hip.ptr(o), _hip.ptr(qn), _hip.ptr(kn), _hip.ptr(kq), _hip.ptr(vv), _hip.ptr(beta), _hip.ptr(decay),
               _hip.ptr(st.pool), st.pool.stride(0), int(state_off), _hip.ptr(st.seq_row0), _hip.ptr(st.seq_cnt),
               _hip.ptr(st.tok_pos), _hip.ptr(st.tok_state), st.seq_row0.shape[0], H, G, d, dv, stream)
     out = torch.empty((n, H * dv), dtype=proj.dtype, device=dev)
