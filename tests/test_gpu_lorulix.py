@@ -491,6 +491,71 @@ def test_other_sizes(tmp_path, dtype, tol, taps):
     assert rel_err(whole[:3], want[:3]) < tol and rel_err(cut[:3], want[:3]) < tol
 
 
+def random_config(rng):
+    """A configuration drawn at random: layer order, head counts and sizes (also ones no kernel is specialised for), taps,
+    experts, which layers borrow keys, which constants are present."""
+    layers, own = [], []
+    for i in range(rng.randint(3, 5)):
+        kind = rng.choice(["none", "dense", "moe", "moe"])
+        if kind == "none":
+            mlp = None
+        elif kind == "dense":
+            mlp = O.dense_mlp(rng.choice([64, 100, 192]), limit=rng.choice([0.8, 2.0, 7.0]))
+        else:
+            experts = rng.choice([2, 4, 8, 16])
+            mlp = O.moe_mlp(rng.choice([16, 48, 80]), experts, rng.randint(1, min(experts, 4)), scale=rng.choice([1.0, 2.5, 0.5]),
+                            shared=rng.choice([None, 32, 72]))
+        r = rng.random()
+        if r < 0.4:
+            kv = rng.choice([1, 2, 3])
+            layers.append(O.delta_layer(heads=kv * rng.choice([1, 2, 3]), kv_heads=kv, dim=rng.choice([16, 24, 32, 64, 128]),
+                                        vdim=rng.choice([16, 40, 64, 128]), conv=rng.choice([1, 2, 3, 4]), mlp=mlp))
+        elif r < 0.75 or not own:
+            kv = rng.choice([1, 2, 4])
+            layers.append(O.attention_layer(heads=kv * rng.choice([1, 2, 3]), kv_heads=kv, dim=rng.choice([16, 32, 48, 64, 128]),
+                                            vdim=rng.choice([16, 32, 64, 128]), scale=rng.choice([0.125, 0.3, 0.08]),
+                                            bias_max=rng.choice([None, 30, 240, 1000]),
+                                            temp=rng.choice([None, (0.5, 64), (0.3, 7), (1.0, 1)]), mlp=mlp))
+            own.append(i)
+        else:
+            j = rng.choice(own)
+            src = layers[j]["mixer"]
+            layers.append(O.attention_layer(heads=src["heads"], kv_heads=src["kv_heads"], dim=src["dim"], vdim=src["vdim"],
+                                            scale=rng.choice([0.125, 0.2]), bias_max=rng.choice([None, 64, 500]),
+                                            temp=rng.choice([None, (0.5, 16)]), kv_from=j, mlp=mlp))
+    return O.make_config(width=rng.choice([64, 96, 160]), vocab=rng.choice([100, 300, 577]), layers=layers,
+                         taps=rng.choice([1, 2, 3, 4]), max_positions=256, eps=rng.choice([1e-5, 1e-6]))
+
+
+@pytest.mark.parametrize("seed", [1, 4, 8, 9])
+def test_random_configurations_in_a_mixed_batch(tmp_path, seed):
+    """Three requests of a randomly drawn model in random portions (single tokens, pairs, page-sized and longer ones) that
+    share steps and sit steps out; every request equals the oracle on the request alone. float32: everywhere."""
+    import random
+    rng = random.Random(seed)
+    cfg = random_config(rng)
+    W = O.make_weights(cfg, seed=seed, bias_rows=rng.choice([8, 13, 32]))
+    reqs = [tokens_for(cfg, n, seed * 10 + i) for i, n in enumerate((120, 37, 64))]
+    wants = [O.forward(cfg, W, t)[0] for t in reqs]
+    model = make_model(tmp_path / "m", cfg, W, "float32", num_blocks=20, max_seqs=3)
+    at, got = [0, 0, 0], [[], [], []]
+    while any(a < len(r) for a, r in zip(at, reqs)):
+        batch = []
+        for i in range(3):
+            if at[i] < len(reqs[i]) and rng.random() < 0.8:
+                c = min(rng.choice([1, 1, 2, 3, 16, 17, 40]), len(reqs[i]) - at[i])
+                batch.append((i, entry(i, reqs[i][at[i]:at[i] + c], at[i])))
+                at[i] += c
+        if batch:
+            lg = model.step([e for _, e in batch])
+            o = 0
+            for i, e in batch:
+                got[i].append(lg[o:o + len(e.tokens)])
+                o += len(e.tokens)
+    for i in range(3):
+        assert rel_err(torch.cat(got[i]), wants[i]) < 5e-5, f"request {i} of {cfg['layers']}"
+
+
 def test_matrix_core_paths_in_the_model(tmp_path):
     """bfloat16 with heads of 64 / 128: the tiled attention with its bias, the expert-stationary kernels, the packed decode
     projections — a prompt in portions and decoded tokens against the oracle on the same (bf16-representable) weights."""
