@@ -597,7 +597,7 @@ int swl_qknorm_full_store_kv(void *qkv, const float *q_w, const float *k_w, void
  * swl_gated_add_rmsnorm: y = m (+ sigmoid(m2_gate[t]) * m2); y *= sigmoid(r + r_bias); x += y / rms(y) * w1; out = x / rms(x)
  * * w2. m NULL: only the output norm, of rows row_idx when given. Per-sequence state: `state` is the base of the state slots
  * (fp32, slot_stride floats apart); tok_state[t] = slot * 2 + parity, tok_start[t] = position of the first token of t's
- * portion. swl_causal_conv_state: out = (h if add_input) + causal convolution of h over time with w [channels, taps] (fp32),
+ * portion. swl_causal_conv_state: out = (h if add_input) + causal convolution of h over time with w [taps, channels] (fp32),
  * the carried inputs at tail_off inside the slot ([2][taps - 1][channels] floats). dtype may be SWL_F32. */
 int swl_gated_add_rmsnorm(float *x, const void *m, const void *m2, const void *m2_gate, int64_t m2_gate_stride,
                           const void *r, int64_t r_stride, const float *r_bias, const float *w1, void *out, const float *w2,

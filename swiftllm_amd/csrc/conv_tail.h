@@ -41,13 +41,12 @@ struct ConvTail {
         return old_tail[static_cast<int64_t>(R - (start - q)) * C + c];
     }
 
-    // sum_j w[c][j] * input(pos - taps + 1 + j); the last tap multiplies the current input `cur`
+    // sum_j w[j][c] * input(pos - taps + 1 + j); w is tap-major [taps, channels], the last tap multiplies the current input
     template <typename T>
     __device__ __forceinline__ float conv(const T *h, int64_t h_stride, const float *w, int c, float cur) const {
-        const float *wc = w + static_cast<int64_t>(c) * taps;
         float a = 0.f;
-        for (int k = taps - 1; k >= 1; --k) a += wc[taps - 1 - k] * at(h, h_stride, c, pos - k);
-        return a + wc[taps - 1] * cur;
+        for (int k = taps - 1; k >= 1; --k) a += w[static_cast<int64_t>(taps - 1 - k) * C + c] * at(h, h_stride, c, pos - k);
+        return a + w[static_cast<int64_t>(taps - 1) * C + c] * cur;
     }
 
     // the portion's last token leaves the sequence's new tail (channel c)
@@ -59,6 +58,82 @@ struct ConvTail {
             if (q < 0) continue;
             new_tail[static_cast<int64_t>(r) * C + c] = q == pos ? cur : at(h, h_stride, c, q);
         }
+    }
+
+    // ---- the same for 8 consecutive channels of 16-bit rows (16-byte loads; c a multiple of 8, rows 16-byte aligned) ----
+    template <typename T>
+    __device__ __forceinline__ void at8(const T *h, int64_t h_stride, int c, int q, float (&v)[8]) const {
+        if (q < 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = 0.f;
+        } else if (q >= start) {
+            const vec8_t<T> x = load8(h + (t - (pos - q)) * h_stride + c);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = to_f(x[j]);
+        } else {
+            const float *p = old_tail + static_cast<int64_t>(R - (start - q)) * C + c;
+            const float4_t a = *reinterpret_cast<const float4_t *>(p), b = *reinterpret_cast<const float4_t *>(p + 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[j] = a[j];
+                v[4 + j] = b[j];
+            }
+        }
+    }
+
+    // same sums in the same order as conv()
+    template <typename T>
+    __device__ __forceinline__ void conv8(const T *h, int64_t h_stride, const float *w, int c, const float (&cur)[8],
+                                          float (&a)[8]) const {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] = 0.f;
+        for (int k = taps - 1; k >= 1; --k) {
+            float v[8];
+            at8(h, h_stride, c, pos - k, v);
+            const float *wk = w + static_cast<int64_t>(taps - 1 - k) * C + c;
+            const float4_t w0 = *reinterpret_cast<const float4_t *>(wk), w1 = *reinterpret_cast<const float4_t *>(wk + 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                a[j] += w0[j] * v[j];
+                a[4 + j] += w1[j] * v[4 + j];
+            }
+        }
+        const float *wl = w + static_cast<int64_t>(taps - 1) * C + c;
+        const float4_t w0 = *reinterpret_cast<const float4_t *>(wl), w1 = *reinterpret_cast<const float4_t *>(wl + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            a[j] += w0[j] * cur[j];
+            a[4 + j] += w1[j] * cur[4 + j];
+        }
+    }
+
+    template <typename T>
+    __device__ __forceinline__ void save8(const T *h, int64_t h_stride, int c, const float (&cur)[8]) const {
+        if (!last || R == 0) return;
+        for (int r = 0; r < R; ++r) {
+            const int q = pos + 1 - R + r;
+            if (q < 0) continue;
+            float v[8];
+            if (q == pos) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = cur[j];
+            } else {
+                at8(h, h_stride, c, q, v);
+            }
+            float *p = new_tail + static_cast<int64_t>(r) * C + c;
+            *reinterpret_cast<float4_t *>(p) = float4_t{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<float4_t *>(p + 4) = float4_t{v[4], v[5], v[6], v[7]};
+        }
+    }
+
+    // whether the 8-channel forms may be used for rows of h (and a state region) laid out like this
+    template <typename T>
+    static __device__ __forceinline__ bool wide_ok(const T *h, int64_t h_stride, const float *w, const float *state,
+                                                   int64_t slot_stride, int64_t tail_off, int channels) {
+        if constexpr (sizeof(T) != 2) return false;
+        return (channels & 7) == 0 && (h_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(h) & 15) == 0 &&
+               (reinterpret_cast<uintptr_t>(w) & 15) == 0 && (reinterpret_cast<uintptr_t>(state) & 15) == 0 &&
+               (slot_stride & 3) == 0 && (tail_off & 3) == 0;
     }
 };
 

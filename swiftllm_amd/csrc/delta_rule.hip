@@ -35,11 +35,28 @@ __global__ __launch_bounds__(kDpThreads) void delta_prep_kernel(
     const int qk = G * d, C = 2 * qk + H * dv;
     const T *row = proj + t * proj_stride;
     const ConvTail tail(state, slot_stride, tail_off, tok_pos, tok_start, tok_state, tok_seq, num_tokens, C, taps, t);
-    for (int c = threadIdx.x; c < C; c += kDpThreads) {
-        const float cur = to_f(row[c]);
-        const float a = tail.conv(proj, proj_stride, conv_w, c, cur);
-        act[c] = a * dr_sigmoid(a);
-        tail.save(proj, proj_stride, c, cur);
+    bool wide = false;
+    if constexpr (sizeof(T) == 2) wide = ConvTail::wide_ok(proj, proj_stride, conv_w, state, slot_stride, tail_off, C);
+    if (wide) {
+        if constexpr (sizeof(T) == 2) {
+            for (int c = threadIdx.x * 8; c < C; c += kDpThreads * 8) {
+                const vec8_t<T> x = load8(row + c);
+                float cur[8], a[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) cur[j] = to_f(x[j]);
+                tail.conv8(proj, proj_stride, conv_w, c, cur, a);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) act[c + j] = a[j] * dr_sigmoid(a[j]);
+                tail.save8(proj, proj_stride, c, cur);
+            }
+        }
+    } else {
+        for (int c = threadIdx.x; c < C; c += kDpThreads) {
+            const float cur = to_f(row[c]);
+            const float a = tail.conv(proj, proj_stride, conv_w, c, cur);
+            act[c] = a * dr_sigmoid(a);
+            tail.save(proj, proj_stride, c, cur);
+        }
     }
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -114,16 +131,14 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float 
     for (int c0 = 0; c0 < cnt; c0 += kDrChunk) {
         const int cn = min(kDrChunk, cnt - c0);
         __syncthreads();        // the previous chunk has been consumed
-        for (int i = threadIdx.x; i < cn * d; i += blockDim.x) {
-            const int j = i / d, e = i - j * d;
+        for (int j = 0; j < cn; ++j) {          // (no divisions by run-time sizes per element)
             const int64_t r = row0 + c0 + j;
-            const int at = j * dp + e + 4 * (e / ds);
-            qs[at] = qn[r * qk + kvh * d + e];
-            ks[at] = kn[r * qk + kvh * d + e];
-        }
-        for (int i = threadIdx.x; i < cn * cpw; i += blockDim.x) {
-            const int j = i / cpw, e = i - j * cpw;
-            vs[i] = vv[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + col0 + e];
+            for (int e = threadIdx.x; e < d; e += blockDim.x) {
+                const int at = j * dp + e + 4 * (EXACT ? e / MAXDS : e / ds);
+                qs[at] = qn[r * qk + kvh * d + e];
+                ks[at] = kn[r * qk + kvh * d + e];
+            }
+            for (int e = threadIdx.x; e < cpw; e += blockDim.x) vs[j * cpw + e] = vv[r * hv + h * dv + col0 + e];
         }
         for (int j = threadIdx.x; j < cn; j += blockDim.x) {
             bs[j] = beta[static_cast<int64_t>(row0 + c0 + j) * H + h];
@@ -161,8 +176,8 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float 
             for (int i = 0; i < MAXDS; ++i) {
                 if (EXACT || i < ds) {
                     s[i] *= g;
-                    sk += s[i] * kr[i];
-                    sq += s[i] * qr[i];
+                    sk = fmaf(s[i], kr[i], sk);
+                    sq = fmaf(s[i], qr[i], sq);
                 }
             }
             sk = dr_group_sum<L>(sk);
@@ -170,8 +185,8 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float 
             const float u = b * (vs[j * cpw + lc] - sk);
 #pragma unroll
             for (int i = 0; i < MAXDS; ++i)
-                if (EXACT || i < ds) s[i] += kr[i] * u;
-            if (l == 0) o[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + col] = sq + u * kq;
+                if (EXACT || i < ds) s[i] = fmaf(kr[i], u, s[i]);
+            if (l == 0) o[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + col] = fmaf(u, kq, sq);
         }
     }
 #pragma unroll
@@ -197,11 +212,12 @@ __global__ __launch_bounds__(256) void gated_head_rmsnorm_kernel(T *out, const f
     }
 }
 
-// lanes per state column: as many as keep at least 8 elements per lane, a power of two that divides dim, at most 16 and at
-// most 1024 threads per workgroup
-inline int dr_lanes(int d, int dv) {
+// lanes per state column: as many as keep at least 16 elements per lane (measured: slices of 8 cost a decode step 1.6x in
+// this kernel, slices of 32 a prompt 1.5x), a power of two that divides dim, at most 16 and at most 1024 threads per
+// workgroup of `cols` columns
+inline int dr_lanes(int d, int cols) {
     int L = 16;
-    while (L > 1 && (d % L || d / L < 8 || static_cast<int64_t>(dv) * L > 1024)) L >>= 1;
+    while (L > 1 && (d % L || d / L < 16 || static_cast<int64_t>(cols) * L > 1024)) L >>= 1;
     return L;
 }
 
@@ -266,12 +282,12 @@ extern "C" int swl_delta_rule(float *o, const float *qn, const float *kn, const 
     if (!o || !qn || !kn || !kq || !vv || !beta || !decay || !state || !seq_row0 || !seq_cnt || !tok_pos || !tok_state)
         return SWL_ERR_BAD_ARG;
     if (vdim > 1024 || num_heads > 65535) return SWL_ERR_UNSUPPORTED;
-    const int L = swl::dr_lanes(dim, vdim);
-    const int ds = dim / L;
     // columns per workgroup: all of them when there are (portion, head) pairs enough to fill the chip (decode batches); a
     // long prompt alone is a sequential walk, so its columns are shared out over more workgroups (down to 16 columns each)
     int cpw = vdim;
     while (static_cast<int64_t>(num_seqs) * num_heads * (vdim / cpw) < 512 && cpw % 2 == 0 && cpw > 16) cpw /= 2;
+    const int L = swl::dr_lanes(dim, cpw);
+    const int ds = dim / L;
     const size_t lds = (static_cast<size_t>(swl::kDrChunk) * (2 * swl::dr_row_floats(dim, L) + cpw + 3)) * sizeof(float);
     if (lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
     const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>(vdim / cpw));

@@ -8,7 +8,7 @@
 //       out = x / rms(x) * w2                  the next sublayer's input (or, with row_idx, the norm of selected rows only)
 //     Statistics, gates and the sum are fp32; m, m2, s, r and out are the compute dtype. Weights arrive as the factor itself
 //     (a loader that stores "weight around zero" adds the one).
-//   swl_causal_conv_state: out[t] = (h[t] if add_input) + sum_j w[c][j] * h[t - taps + 1 + j] per channel over the tokens of
+//   swl_causal_conv_state: out[t] = (h[t] if add_input) + sum_j w[j][c] * h[t - taps + 1 + j] per channel (w tap-major) over the tokens of
 //     one sequence, for any cut of the sequence into steps: inputs of earlier steps come from the sequence's state slot,
 //     which keeps the last taps - 1 inputs. The tail is double-buffered: a step reads buffer `parity` and the workgroup of
 //     a portion's last token writes the other one, so no launch reads what it writes.
@@ -75,6 +75,24 @@ __global__ __launch_bounds__(kRsThreads) void causal_conv_state_kernel(
     int64_t num_tokens, int C, int taps, int add_input) {
     const int64_t t = blockIdx.x;
     const ConvTail tail(state, slot_stride, tail_off, tok_pos, tok_start, tok_state, tok_seq, num_tokens, C, taps, t);
+    if constexpr (sizeof(T) == 2) {
+        if (ConvTail::wide_ok(h, h_stride, w, state, slot_stride, tail_off, C) && (out_stride & 7) == 0 &&
+            (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+            for (int c = threadIdx.x * 8; c < C; c += kRsThreads * 8) {
+                const vec8_t<T> x = load8(h + t * h_stride + c);
+                float cur[8], a[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) cur[j] = to_f(x[j]);
+                tail.conv8(h, h_stride, w, c, cur, a);
+                vec8_t<T> o;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = to_t<T>(add_input ? a[j] + cur[j] : a[j]);
+                store8(out + t * out_stride + c, o);
+                tail.save8(h, h_stride, c, cur);
+            }
+            return;
+        }
+    }
     for (int c = threadIdx.x; c < C; c += kRsThreads) {
         const float cur = to_f(h[t * h_stride + c]);
         float a = tail.conv(h, h_stride, w, c, cur);

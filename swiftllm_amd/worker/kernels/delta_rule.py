@@ -8,14 +8,15 @@ from .rms_stream import StateRef
 
 def delta_rule_mixer(proj: torch.Tensor, conv_w: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                      norm_w: torch.Tensor, st: StateRef, tail_off: int, state_off: int, mixer, eps: float) -> torch.Tensor:
-    """proj [T, q | k | v | gate | b | a] (one fused projection) -> [T, heads * vdim] in proj's dtype: short convolutions +
+    """proj [T, q | k | v | gate | b | a] (one fused projection) -> [T, heads * vdim] in proj's dtype: short convolutions
+    (conv_w tap-major [taps, q | k | v channels]) +
     SiLU, unit q / k, the token-by-token recurrence on the fp32 state [heads, dim, vdim] at `state_off` inside each
     sequence's slot, then per head o / rms(o) * norm_w * silu(gate)."""
     _hip.require_gpu_tensor(proj, "proj")
     n = proj.shape[0]
     H, G, d, dv = mixer.num_heads, mixer.num_kv_heads, mixer.head_dim, mixer.value_dim
     assert proj.stride(1) == 1 and proj.shape[1] == mixer.proj_size
-    assert conv_w.dtype == torch.float32 and conv_w.is_contiguous() and conv_w.shape == (mixer.conv_channels, mixer.conv_taps)
+    assert conv_w.dtype == torch.float32 and conv_w.is_contiguous() and conv_w.shape == (mixer.conv_taps, mixer.conv_channels)
     assert a_log.dtype == dt_bias.dtype == norm_w.dtype == torch.float32 and a_log.numel() == dt_bias.numel() == H
     assert norm_w.numel() == dv
     dev, f32 = proj.device, torch.float32

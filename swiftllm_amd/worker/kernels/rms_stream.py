@@ -44,14 +44,14 @@ class StateRef:
 
 
 def causal_conv_state(h: torch.Tensor, w: torch.Tensor, st: StateRef, tail_off: int, add_input: bool) -> torch.Tensor:
-    """(h +) causal convolution of h over time per channel; w fp32 [channels, taps]; the last taps - 1 inputs of every
-    sequence are carried at `tail_off` inside its state slot."""
+    """(h +) causal convolution of h over time per channel; w fp32, tap-major [taps, channels] (the last row multiplies the
+    current token); the last taps - 1 inputs of every sequence are carried at `tail_off` inside its state slot."""
     _hip.require_gpu_tensor(h, "h")
     n, c = h.shape
-    assert h.stride(1) == 1 and w.dtype == torch.float32 and w.is_contiguous() and w.shape[0] == c
+    assert h.stride(1) == 1 and w.dtype == torch.float32 and w.is_contiguous() and w.shape[1] == c
     out = torch.empty((n, c), dtype=h.dtype, device=h.device)
     _hip.call("swl_causal_conv_state", _hip.ptr(out), out.stride(0), _hip.ptr(h), h.stride(0), _hip.ptr(w),
               _hip.ptr(st.pool), st.pool.stride(0), int(tail_off), _hip.ptr(st.tok_pos), _hip.ptr(st.tok_start),
-              _hip.ptr(st.tok_state), _hip.ptr(st.tok_seq), n, c, w.shape[1], 1 if add_input else 0,
+              _hip.ptr(st.tok_state), _hip.ptr(st.tok_seq), n, c, w.shape[0], 1 if add_input else 0,
               _hip.dtype_code3(h.dtype), _hip.stream())
     return out

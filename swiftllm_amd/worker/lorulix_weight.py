@@ -43,7 +43,7 @@ class LorulixLayerWeight:
         for k in ("1", "2") if lcfg.mlp is not None else ("1",):
             setattr(self, "norm" + k, one_plus("norm" + k, (w,)))
             setattr(self, "norm" + k + "b", one_plus("norm" + k + "b", (w,)))
-            setattr(self, "canon" + k, f32("canon" + k, (w, cfg.canon_taps)))
+            setattr(self, "canon" + k, f32("canon" + k, (w, cfg.canon_taps)).t().contiguous())      # tap-major
             setattr(self, "rg" + k, mat("rg" + k, (w, w)))
             setattr(self, "rg" + k + "_b", f32("rg" + k + ".b", (w,)))
         if lcfg.type == "attention":
@@ -66,7 +66,7 @@ class LorulixLayerWeight:
                                    mat("mix.v", (mx.v_size, w)), mat("mix.g", (mx.v_size, w)), mat("mix.b", (H, w)),
                                    mat("mix.a", (H, w))), dim=0).contiguous()
             self.conv = torch.cat((f32("mix.q.conv", (mx.qk_size, t)), f32("mix.k.conv", (mx.qk_size, t)),
-                                   f32("mix.v.conv", (mx.v_size, t))), dim=0).contiguous()
+                                   f32("mix.v.conv", (mx.v_size, t))), dim=0).t().contiguous()     # tap-major
             self.a_log = f32("mix.A_log", (H,))
             self.dt_bias = f32("mix.dt_bias", (H,))
             self.out_norm = f32("mix.norm", (mx.value_dim,))

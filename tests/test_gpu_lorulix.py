@@ -175,7 +175,7 @@ def test_causal_convolution_in_portions_and_reused_slots(taps):
             portions = [(pair[s], start, cnt) for s, start, cnt in step]
             st = slots.ref(portions)
             h = torch.cat([hs[s][start:start + cnt] for s, start, cnt in portions]).cuda()
-            out = causal_conv_state(h, w.cuda(), st, slots.off[0], add_input=True).cpu()
+            out = causal_conv_state(h, w.t().contiguous().cuda(), st, slots.off[0], add_input=True).cpu()
             at = 0
             for s, start, cnt in portions:
                 got[s].append(out[at:at + cnt])
@@ -201,7 +201,7 @@ def test_delta_rule_in_portions(H, G, d, e, conv, n, dtype):
          "v.conv": torch.randn(H * e, conv, generator=g) * 0.6, "A_log": torch.randn(H, generator=g) * 0.5,
          "dt_bias": torch.randn(H, generator=g) * 0.5, "norm": 1 + 0.2 * torch.randn(e, generator=g)}
     Wd = {k: v.double() for k, v in W.items()}
-    conv_w = torch.cat((W["q.conv"], W["k.conv"], W["v.conv"])).cuda()
+    conv_w = torch.cat((W["q.conv"], W["k.conv"], W["v.conv"])).t().contiguous().cuda()     # tap-major
     lengths = [n, 11]
     projs = [(torch.randn(m, mc.proj_size, generator=g) * 1.5).to(dtype) for m in lengths]
     want = []
