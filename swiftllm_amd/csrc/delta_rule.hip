@@ -20,7 +20,7 @@
 namespace swl {
 
 constexpr int kDpThreads = 256;
-constexpr int kDrChunk = 16;        // tokens staged per round
+constexpr int kDrChunk = 16;        // tokens staged at a time
 
 __device__ __forceinline__ float dr_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 

@@ -294,7 +294,7 @@ def test_attention_with_distance_bias(H, G, d, e, n):
     assert (got - want).abs().max() < 2e-5
 
 
-@pytest.mark.parametrize("H,G,d,e,n", [(4, 2, 64, 64, 150), (8, 2, 128, 64, 90), (3, 1, 64, 128, 37), (16, 4, 128, 128, 64)])
+@pytest.mark.parametrize("H,G,d,e,n", [(4, 1, 64, 64, 150), (8, 2, 128, 64, 90), (3, 1, 64, 128, 37), (16, 4, 128, 128, 64)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_matrix_core_attention_with_distance_bias(H, G, d, e, n, dtype):
     g = torch.Generator().manual_seed(n)
@@ -332,7 +332,7 @@ def test_a_far_key_among_hundreds_is_found(tiled, dtype, d):
     qkv[13, H * d:(H + G) * d] = 4 * u
     qkv[-6:, :H * d] = 4 * u.repeat(H)
     rel = torch.randn(10, H, generator=g)
-    got, want = _attention_case(H, G, d, e, n, dtype, rel, (0.5, 64), qkv, tiled, chunks=(397, 1))
+    got, want = _attention_case(H, G, d, e, n, dtype, rel, (0.5, 48), qkv, tiled, chunks=(397, 1))
     v13 = qkv[13, (H + G) * d:].to(dtype).double()
     assert (want[-1, :e] - v13).abs().max() < 0.2 * float(v13.abs().max())      # the oracle itself attends there
     assert (got - want).abs().max() < (2e-5 if dtype == torch.float32 else 3e-2)
@@ -343,7 +343,7 @@ def test_a_far_key_among_hundreds_is_found(tiled, dtype, d):
 def test_router_and_squared_relu_experts(experts, top, shared, n):
     from swiftllm_amd.worker.kernels.moe import moe_experts_relu2, moe_route_scores
     g = torch.Generator().manual_seed(experts)
-    w, ff, scale = 48, 32, 2.5
+    w, ff, scale = 48, 32, 1.7
     h = torch.randn(n, w, generator=g)
     W = {"router": torch.randn(experts, w, generator=g)}
     for x in range(experts):
@@ -500,10 +500,10 @@ def random_config(rng):
         if kind == "none":
             mlp = None
         elif kind == "dense":
-            mlp = O.dense_mlp(rng.choice([64, 100, 192]), limit=rng.choice([0.8, 2.0, 7.0]))
+            mlp = O.dense_mlp(rng.choice([64, 100, 176]), limit=rng.choice([0.8, 1.7, 7.0]))
         else:
             experts = rng.choice([2, 4, 8, 16])
-            mlp = O.moe_mlp(rng.choice([16, 48, 80]), experts, rng.randint(1, min(experts, 4)), scale=rng.choice([1.0, 2.5, 0.5]),
+            mlp = O.moe_mlp(rng.choice([16, 48, 80]), experts, rng.randint(1, min(experts, 4)), scale=rng.choice([1.0, 2.0, 0.5]),
                             shared=rng.choice([None, 32, 72]))
         r = rng.random()
         if r < 0.4:
@@ -513,15 +513,15 @@ def random_config(rng):
         elif r < 0.75 or not own:
             kv = rng.choice([1, 2, 4])
             layers.append(O.attention_layer(heads=kv * rng.choice([1, 2, 3]), kv_heads=kv, dim=rng.choice([16, 32, 48, 64, 128]),
-                                            vdim=rng.choice([16, 32, 64, 128]), scale=rng.choice([0.125, 0.3, 0.08]),
-                                            bias_max=rng.choice([None, 30, 240, 1000]),
-                                            temp=rng.choice([None, (0.5, 64), (0.3, 7), (1.0, 1)]), mlp=mlp))
+                                            vdim=rng.choice([16, 32, 64, 128]), scale=rng.choice([0.11, 0.3, 0.08]),
+                                            bias_max=rng.choice([None, 30, 200, 1000]),
+                                            temp=rng.choice([None, (0.5, 48), (0.3, 7), (1.0, 1)]), mlp=mlp))
             own.append(i)
         else:
             j = rng.choice(own)
             src = layers[j]["mixer"]
             layers.append(O.attention_layer(heads=src["heads"], kv_heads=src["kv_heads"], dim=src["dim"], vdim=src["vdim"],
-                                            scale=rng.choice([0.125, 0.2]), bias_max=rng.choice([None, 64, 500]),
+                                            scale=rng.choice([0.15, 0.2]), bias_max=rng.choice([None, 64, 500]),
                                             temp=rng.choice([None, (0.5, 16)]), kv_from=j, mlp=mlp))
     return O.make_config(width=rng.choice([64, 96, 160]), vocab=rng.choice([100, 300, 577]), layers=layers,
                          taps=rng.choice([1, 2, 3, 4]), max_positions=256, eps=rng.choice([1e-5, 1e-6]))
@@ -559,9 +559,9 @@ def test_random_configurations_in_a_mixed_batch(tmp_path, seed):
 def test_matrix_core_paths_in_the_model(tmp_path):
     """bfloat16 with heads of 64 / 128: the tiled attention with its bias, the expert-stationary kernels, the packed decode
     projections — a prompt in portions and decoded tokens against the oracle on the same (bf16-representable) weights."""
-    layers = [O.attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, bias_max=120, mlp=O.moe_mlp(64, 8, 2, shared=64)),
+    layers = [O.attention_layer(heads=8, kv_heads=2, dim=64, vdim=128, bias_max=120, mlp=O.moe_mlp(64, 8, 2, shared=64)),
               O.delta_layer(heads=4, kv_heads=2, dim=64, vdim=64, conv=4, mlp=O.dense_mlp(256)),
-              O.attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, bias_max=120, kv_from=0, mlp=O.moe_mlp(64, 8, 2))]
+              O.attention_layer(heads=8, kv_heads=2, dim=64, vdim=128, bias_max=120, kv_from=0, mlp=O.moe_mlp(64, 8, 2))]
     cfg = O.make_config(width=128, vocab=160, layers=layers, max_positions=256)
     W = O.make_weights(cfg, seed=5, bias_rows=16)
     toks = tokens_for(cfg, 140, 6)
