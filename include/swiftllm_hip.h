@@ -611,7 +611,8 @@ int swl_causal_conv_state(void *out, int64_t out_stride, const void *h, int64_t 
 /* ---- gated delta rule (csrc/delta_rule.hip) --------------------------------------------------------------------------------
  * swl_delta_prep: proj rows [q | k | v | gate | b | a] -> qn, kn [T, qk heads * dim], kq [T, qk heads] (their dot
  * products), vv [T, heads * vdim], beta, decay
- * [T, heads], all fp32 (convolution + SiLU, unit norms, sigmoid, exp(-exp(A_log) softplus(a + dt_bias))).
+ * [T, heads], all fp32 (convolution + SiLU with conv_w tap-major [taps, q | k | v channels], unit norms, sigmoid,
+ * exp(-exp(A_log) softplus(a + dt_bias))).
  * swl_delta_rule: o[T, heads * vdim] (fp32) and the states [heads, dim, vdim] at s_off inside the slots, one portion per
  * (seq_row0, seq_cnt) entry. swl_gated_head_rmsnorm: out = o / rms(o over vdim) * w[vdim] * silu(gate). */
 int swl_delta_prep(float *qn, float *kn, float *kq, float *vv, float *beta, float *decay, const void *proj, int64_t proj_stride,

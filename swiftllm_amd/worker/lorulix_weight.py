@@ -8,8 +8,9 @@ What the loader does with them:
   * projection matrices go to the device in the compute dtype; matrices that multiply the same input are concatenated into
     one (attention: q | k | v; delta rule: q | k | v | output gate | beta | decay; dense feed-forward: gate | up; shared
     expert: up | its per-token gate), experts are stacked ([experts, ff, width], [experts, width, ff]);
-  * everything that enters fp32 arithmetic — norm weights (stored around zero: kept as 1 + w), convolution taps, gate
-    biases, q/k norm weights, the recurrence's A_log / dt_bias / output norm, the router — is kept in fp32 (exact: the
+  * everything that enters fp32 arithmetic — norm weights (stored around zero: kept as 1 + w), convolution taps (stored
+    [channels, taps], kept tap-major [taps, channels] so that a lane reads the taps of 8 channels with two 16-byte loads),
+    gate biases, q/k norm weights, the recurrence's A_log / dt_bias / output norm, the router — is kept in fp32 (exact: the
     checkpoint holds bfloat16);
   * the learned distance bias [rows, heads] is expanded once, on the host in float64, to a table [heads, positions] indexed
     by distance, so that no kernel evaluates the bucket function.
