@@ -131,14 +131,36 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float 
     for (int c0 = 0; c0 < cnt; c0 += kDrChunk) {
         const int cn = min(kDrChunk, cnt - c0);
         __syncthreads();        // the previous chunk has been consumed
-        for (int j = 0; j < cn; ++j) {          // (no divisions by run-time sizes per element)
-            const int64_t r = row0 + c0 + j;
-            for (int e = threadIdx.x; e < d; e += blockDim.x) {
-                const int at = j * dp + e + 4 * (EXACT ? e / MAXDS : e / ds);
-                qs[at] = qn[r * qk + kvh * d + e];
-                ks[at] = kn[r * qk + kvh * d + e];
+        // all of a chunk's loads are issued before the first one is waited for: one memory round trip per chunk (issued
+        // load by load, with an LDS store between two loads, the round trips of a chunk lined up one after the other and
+        // were most of the kernel's time)
+        for (int e = threadIdx.x; e < d; e += blockDim.x) {
+            float tq[kDrChunk], tk[kDrChunk];
+            const float *qsrc = qn + static_cast<int64_t>(row0 + c0) * qk + kvh * d + e;
+            const float *ksrc = kn + static_cast<int64_t>(row0 + c0) * qk + kvh * d + e;
+#pragma unroll
+            for (int j = 0; j < kDrChunk; ++j) {
+                const int jj = min(j, cn - 1);      // (rows past the chunk's end re-read its last row: never stored)
+                tq[j] = qsrc[static_cast<int64_t>(jj) * qk];
+                tk[j] = ksrc[static_cast<int64_t>(jj) * qk];
             }
-            for (int e = threadIdx.x; e < cpw; e += blockDim.x) vs[j * cpw + e] = vv[r * hv + h * dv + col0 + e];
+            const int at = e + 4 * (EXACT ? e / MAXDS : e / ds);
+#pragma unroll
+            for (int j = 0; j < kDrChunk; ++j) {
+                if (j < cn) {
+                    qs[j * dp + at] = tq[j];
+                    ks[j * dp + at] = tk[j];
+                }
+            }
+        }
+        for (int e = threadIdx.x; e < cpw; e += blockDim.x) {
+            float tv[kDrChunk];
+            const float *vsrc = vv + static_cast<int64_t>(row0 + c0) * hv + h * dv + col0 + e;
+#pragma unroll
+            for (int j = 0; j < kDrChunk; ++j) tv[j] = vsrc[static_cast<int64_t>(min(j, cn - 1)) * hv];
+#pragma unroll
+            for (int j = 0; j < kDrChunk; ++j)
+                if (j < cn) vs[j * cpw + e] = tv[j];
         }
         for (int j = threadIdx.x; j < cn; j += blockDim.x) {
             bs[j] = beta[static_cast<int64_t>(row0 + c0 + j) * H + h];
