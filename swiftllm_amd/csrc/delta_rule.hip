@@ -12,7 +12,8 @@
 //                    two partial dot products (S^T k, S^T q) through DPP and o = S^T q + u (k . q, from the prep) needs no second
 //                    pass over the state. q, k, v, beta, g of 16 tokens at a time are staged in LDS. The token loop is
 //                    sequential whatever the cut of the sequence into steps: the same operations in the same order. When
-//                    a step has few (portion, head) pairs the columns of a head are shared out over several workgroups.
+//                    a step has few (portion, head) pairs the columns of a head are shared out over several workgroups. A
+//                    wave of loaders stages the next 16 tokens into a second LDS buffer while the others walk the current ones.
 //   swl_gated_head_rmsnorm: out = o / rms(o over vdim) * w * silu(gate), per head.
 #include "swl_common.h"
 #include "conv_tail.h"
@@ -101,48 +102,49 @@ __host__ __device__ inline int dr_row_floats(int d, int L) { return d + 4 * L; }
 
 template <int MAXDS, int L, bool EXACT>
 __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float *qn, const float *kn, const float *kqn,
-                                                          const float *vv,
-                                                          const float *beta, const float *decay, float *state,
-                                                          int64_t slot_stride, int64_t s_off, const int32_t *seq_row0,
-                                                          const int32_t *seq_cnt, const int32_t *tok_pos,
-                                                          const int32_t *tok_state, int H, int G, int d, int dv, int cpw) {
+                                                          const float *vv, const float *beta, const float *decay,
+                                                          float *state, int64_t slot_stride, int64_t s_off,
+                                                          const int32_t *seq_row0, const int32_t *seq_cnt,
+                                                          const int32_t *tok_pos, const int32_t *tok_state, int H, int G,
+                                                          int d, int dv, int cpw, int nload) {
+    // nload > 0: the last nload threads of the workgroup only LOAD — they stage chunk c + 1 into the other LDS buffer while
+    // the first cpw * L threads walk the tokens of chunk c, one barrier per chunk. nload = 0: everybody stages, then walks.
     extern __shared__ float lds[];
     const int dp = dr_row_floats(d, L);
-    float *qs = lds;                        // [chunk][dp]
-    float *ks = qs + kDrChunk * dp;         // [chunk][dp]
-    float *vs = ks + kDrChunk * dp;         // [chunk][cpw]
-    float *bs = vs + kDrChunk * cpw;        // [chunk]
-    float *gs = bs + kDrChunk;              // [chunk]
-    float *kqs = gs + kDrChunk;             // [chunk] k . q of the token's (normed) q / k head
+    const int buf_floats = kDrChunk * (2 * dp + cpw + 3);
     const int seq = blockIdx.x, h = blockIdx.y;
     const int col0 = blockIdx.z * cpw;      // this workgroup's columns of the state (independent recurrences)
     const int row0 = seq_row0[seq], cnt = seq_cnt[seq];
     const int kvh = h / (H / G);
-    const int lc = threadIdx.x / L, l = threadIdx.x % L;
+    const int ncomp = static_cast<int>(blockDim.x) - nload;
+    const bool computes = static_cast<int>(threadIdx.x) < ncomp;
+    const int lc = computes ? threadIdx.x / L : 0, l = threadIdx.x % L;
     const int col = col0 + lc;
     const int ds = EXACT ? MAXDS : d / L, i0 = l * ds;      // (EXACT: the slice fills the register array, no predicates)
+    const int qk = G * d, hv = H * dv;
     float *S = state + static_cast<int64_t>(tok_state[row0] >> 1) * slot_stride + s_off + static_cast<int64_t>(h) * d * dv;
     float s[MAXDS];
     const bool fresh = tok_pos[row0] == 0;      // a sequence starts from the zero state whatever the slot held
 #pragma unroll
-    for (int i = 0; i < MAXDS; ++i) s[i] = (i < ds && !fresh) ? S[static_cast<int64_t>(i0 + i) * dv + col] : 0.f;
-    const int qk = G * d, hv = H * dv;
+    for (int i = 0; i < MAXDS; ++i) s[i] = (computes && i < ds && !fresh) ? S[static_cast<int64_t>(i0 + i) * dv + col] : 0.f;
     const bool quads = EXACT || (ds & 3) == 0;  // 16-byte LDS reads
-    for (int c0 = 0; c0 < cnt; c0 += kDrChunk) {
+
+    // Stage the chunk at c0 into `buf` with threads sid, sid + sn, ...: all of the chunk's loads are issued before the first
+    // one is waited for — one memory round trip per chunk (load by load, with an LDS store between two loads, the round
+    // trips of a chunk line up one after the other).
+    auto stage = [&](int c0, float *buf, int sid, int sn) {
         const int cn = min(kDrChunk, cnt - c0);
-        __syncthreads();        // the previous chunk has been consumed
-        // all of a chunk's loads are issued before the first one is waited for: one memory round trip per chunk (issued
-        // load by load, with an LDS store between two loads, the round trips of a chunk lined up one after the other and
-        // were most of the kernel's time)
-        for (int e = threadIdx.x; e < d; e += blockDim.x) {
+        float *qs = buf, *ks = qs + kDrChunk * dp, *vs = ks + kDrChunk * dp, *bs = vs + kDrChunk * cpw;
+        float *gs = bs + kDrChunk, *kqs = gs + kDrChunk;
+        for (int e = sid; e < d; e += sn) {
             float tq[kDrChunk], tk[kDrChunk];
             const float *qsrc = qn + static_cast<int64_t>(row0 + c0) * qk + kvh * d + e;
             const float *ksrc = kn + static_cast<int64_t>(row0 + c0) * qk + kvh * d + e;
 #pragma unroll
             for (int j = 0; j < kDrChunk; ++j) {
-                const int jj = min(j, cn - 1);      // (rows past the chunk's end re-read its last row: never stored)
-                tq[j] = qsrc[static_cast<int64_t>(jj) * qk];
-                tk[j] = ksrc[static_cast<int64_t>(jj) * qk];
+                const int64_t jj = min(j, cn - 1);      // (rows past the chunk's end re-read its last row: never stored)
+                tq[j] = qsrc[jj * qk];
+                tk[j] = ksrc[jj * qk];
             }
             const int at = e + 4 * (EXACT ? e / MAXDS : e / ds);
 #pragma unroll
@@ -153,7 +155,7 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float 
                 }
             }
         }
-        for (int e = threadIdx.x; e < cpw; e += blockDim.x) {
+        for (int e = sid; e < cpw; e += sn) {
             float tv[kDrChunk];
             const float *vsrc = vv + static_cast<int64_t>(row0 + c0) * hv + h * dv + col0 + e;
 #pragma unroll
@@ -162,12 +164,18 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float 
             for (int j = 0; j < kDrChunk; ++j)
                 if (j < cn) vs[j * cpw + e] = tv[j];
         }
-        for (int j = threadIdx.x; j < cn; j += blockDim.x) {
+        for (int j = sid; j < cn; j += sn) {
             bs[j] = beta[static_cast<int64_t>(row0 + c0 + j) * H + h];
             gs[j] = decay[static_cast<int64_t>(row0 + c0 + j) * H + h];
             kqs[j] = kqn[static_cast<int64_t>(row0 + c0 + j) * G + kvh];
         }
-        __syncthreads();
+    };
+
+    // Walk the tokens of the chunk at c0 (staged in `buf`): the sequential part.
+    auto walk = [&](int c0, const float *buf) {
+        const int cn = min(kDrChunk, cnt - c0);
+        const float *qs = buf, *ks = qs + kDrChunk * dp, *vs = ks + kDrChunk * dp, *bs = vs + kDrChunk * cpw;
+        const float *gs = bs + kDrChunk, *kqs = gs + kDrChunk;
 #pragma unroll 2
         for (int j = 0; j < cn; ++j) {
             const float g = gs[j], b = bs[j], kq = kqs[j];
@@ -210,7 +218,26 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(float *o, const float 
                 if (EXACT || i < ds) s[i] = fmaf(kr[i], u, s[i]);
             if (l == 0) o[static_cast<int64_t>(row0 + c0 + j) * hv + h * dv + col] = fmaf(u, kq, sq);
         }
+    };
+
+    if (nload > 0) {
+        if (!computes) stage(0, lds, static_cast<int>(threadIdx.x) - ncomp, nload);
+        __syncthreads();
+        int c = 0;
+        for (int c0 = 0; c0 < cnt; c0 += kDrChunk, ++c) {
+            if (computes) walk(c0, lds + (c & 1) * buf_floats);
+            else if (c0 + kDrChunk < cnt) stage(c0 + kDrChunk, lds + ((c + 1) & 1) * buf_floats, static_cast<int>(threadIdx.x) - ncomp, nload);
+            __syncthreads();    // chunk c has been walked and chunk c + 1 is in place
+        }
+    } else {
+        for (int c0 = 0; c0 < cnt; c0 += kDrChunk) {
+            __syncthreads();    // the previous chunk has been consumed
+            stage(c0, lds, threadIdx.x, blockDim.x);
+            __syncthreads();
+            walk(c0, lds);
+        }
     }
+    if (!computes) return;
 #pragma unroll
     for (int i = 0; i < MAXDS; ++i)
         if (i < ds) S[static_cast<int64_t>(i0 + i) * dv + col] = s[i];
@@ -234,9 +261,9 @@ __global__ __launch_bounds__(256) void gated_head_rmsnorm_kernel(T *out, const f
     }
 }
 
-// lanes per state column: as many as keep at least 16 elements per lane (measured: slices of 8 cost a decode step 1.6x in
-// this kernel, slices of 32 a prompt 1.5x), a power of two that divides dim, at most 16 and at most 1024 threads per
-// workgroup of `cols` columns
+// lanes per state column: as many as keep at least 16 elements per lane (measured: slices of 8 do not shorten a prompt's walk
+// and cost a decode launch 1.6x, slices of 32 cost a prompt 1.5x), a power of two that divides dim, at most 16 and at most
+// 1024 threads per workgroup of `cols` columns
 inline int dr_lanes(int d, int cols) {
     int L = 16;
     while (L > 1 && (d % L || d / L < 16 || static_cast<int64_t>(cols) * L > 1024)) L >>= 1;
@@ -247,10 +274,10 @@ template <int L>
 int launch_dr(int ds, dim3 grid, dim3 block, size_t lds, hipStream_t s, float *o, const float *qn, const float *kn,
               const float *kq, const float *vv, const float *beta, const float *decay, float *state, int64_t slot_stride, int64_t s_off,
               const int32_t *seq_row0, const int32_t *seq_cnt, const int32_t *tok_pos, const int32_t *tok_state, int H,
-              int G, int d, int dv, int cpw) {
+              int G, int d, int dv, int cpw, int nload) {
 #define SWL_DR_LAUNCH1(M, X)                                                                                                 \
     hipLaunchKernelGGL((delta_rule_kernel<M, L, X>), grid, block, lds, s, o, qn, kn, kq, vv, beta, decay, state, slot_stride, \
-                       s_off, seq_row0, seq_cnt, tok_pos, tok_state, H, G, d, dv, cpw)
+                       s_off, seq_row0, seq_cnt, tok_pos, tok_state, H, G, d, dv, cpw, nload)
 #define SWL_DR_LAUNCH(M)                   \
     if (ds == M) SWL_DR_LAUNCH1(M, true);  \
     else SWL_DR_LAUNCH1(M, false)
@@ -310,14 +337,17 @@ extern "C" int swl_delta_rule(float *o, const float *qn, const float *kn, const 
     while (static_cast<int64_t>(num_seqs) * num_heads * (vdim / cpw) < 512 && cpw % 2 == 0 && cpw > 16) cpw /= 2;
     const int L = swl::dr_lanes(dim, cpw);
     const int ds = dim / L;
-    const size_t lds = (static_cast<size_t>(swl::kDrChunk) * (2 * swl::dr_row_floats(dim, L) + cpw + 3)) * sizeof(float);
-    if (lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    const size_t one = (static_cast<size_t>(swl::kDrChunk) * (2 * swl::dr_row_floats(dim, L) + cpw + 3)) * sizeof(float);
+    if (one > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    // a wave of loaders and a second LDS buffer when both fit and there is more than one chunk's worth of tokens to gain from
+    const int nload = (cpw * L + 64 <= 1024 && 2 * one <= 64 * 1024) ? 64 : 0;
+    const size_t lds = nload ? 2 * one : one;
     const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>(vdim / cpw));
-    const dim3 block(static_cast<unsigned>(cpw * L));
+    const dim3 block(static_cast<unsigned>(cpw * L + nload));
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define SWL_DR_L(LL)                                                                                                         \
     case LL: return swl::launch_dr<LL>(ds, grid, block, lds, s, o, qn, kn, kq, vv, beta, decay, state, slot_stride, s_off,       \
-                                       seq_row0, seq_cnt, tok_pos, tok_state, num_heads, num_qk_heads, dim, vdim, cpw)
+                                       seq_row0, seq_cnt, tok_pos, tok_state, num_heads, num_qk_heads, dim, vdim, cpw, nload)
     switch (L) {
         SWL_DR_L(1);
         SWL_DR_L(2);
